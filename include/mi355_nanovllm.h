@@ -658,9 +658,9 @@ int mi_gemm_any(const float* x, int64_t ldx, const void* w, int w_dtype, float* 
 int mi_gemm_any_grouped(const float* x, int64_t ldx, const int32_t* x_rows, const void* w, const void* w2, int w_dtype,
                         const int32_t* group_offsets, int n_groups, int rows_per_group_max, float* y, int64_t ldy,
                         const int32_t* y_rows, int N, int K, int exact, mi_stream stream);
-/* out[i] = table[ids[i]] widened to fp32. */
+/* out[i] = table[ids[i]] widened to fp32, times scale. */
 int mi_embedding_f32(const int64_t* ids, const void* table, int table_dtype, float* out, int n, int width, int vocab,
-                     mi_stream stream);
+                     float scale, mi_stream stream);
 /* LayerNorm (mean and mean squared deviation in fp32, eps inside the root, weight and bias) of each row of y;
  * add_to_out != 0: out += LN(y) (a residual stream whose norm sits on the sublayer's output). */
 int mi_layernorm_f32(const float* y, int64_t ldy, const float* w, const float* b, float* out, int64_t ldo, int rows,
@@ -686,6 +686,11 @@ int mi_swa_attention(const float* q, int64_t ldq, const void* k_cache, const voi
 int mi_causal_conv_silu(const float* x, int64_t ldx, const float* w, int taps, const float* state, const int32_t* cu_q,
                         const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int rows, int channels, float* y,
                         int64_t ldy, mi_stream stream);
+/* The general form: silu != 0: y = silu(conv(x)), else y = conv(x); add_input != 0: y += x (a convolution beside the
+ * identity: what a sublayer reads is x + conv(x)). */
+int mi_causal_conv(const float* x, int64_t ldx, const float* w, int taps, const float* state, const int32_t* cu_q,
+                   const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int rows, int channels, int silu,
+                   int add_input, float* y, int64_t ldy, mi_stream stream);
 int mi_causal_conv_state(const float* x, int64_t ldx, int taps, float* state, const int32_t* cu_q,
                          const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int channels, mi_stream stream);
 /* Floats of recurrent state one sequence slot holds for mi_channel_delta (the kernel's own thread-order layout), or
@@ -703,11 +708,16 @@ int mi_channel_delta(const float* qkv, int64_t ld, int q_off, int k_off, int v_o
                      const float* a_log, const float* gate_pre, int64_t ld_gate, const float* norm_w, float* state,
                      const int32_t* cu_q, const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int n_rows, int H,
                      int G, int D, int Dv, float eps, float* workspace, float* out, int64_t ldo, mi_stream stream);
-/* Router with expert groups: scores = softmax(logits) over n_outputs; choice = scores + correction; only the
- * `keep` of `n_groups` equal groups of neighbours with the largest best choice are eligible; ids = the top_k
- * eligible outputs by choice (descending), weights = their scores (not renormalised).  n_outputs <= 512. */
+#define MI_ROUTE_SOFTMAX 0    /* scores = softmax(logits) over n_outputs */
+#define MI_ROUTE_SIGMOID 1    /* scores = sigmoid(logits), each output for itself */
+#define MI_ROUTE_GROUP_MAX  0 /* a group's value: its largest choice score */
+#define MI_ROUTE_GROUP_TOP2 1 /* the sum of its two largest (a group of one output: that one's) */
+/* Router with expert groups: scores by score_kind; choice = scores + correction; only the `keep` of `n_groups` equal
+ * groups of neighbours with the largest values (group_kind) are eligible; ids = the top_k eligible outputs by choice
+ * (descending; equal: the lower index), weights = their scores (not renormalised).  n_outputs <= 512. */
 int mi_route_grouped(const float* logits, int64_t ld, const float* correction, int n_tokens, int n_outputs, int top_k,
-                     int n_groups, int keep, int32_t* ids, float* weights, mi_stream stream);
+                     int n_groups, int keep, int score_kind, int group_kind, int32_t* ids, float* weights,
+                     mi_stream stream);
 /* out[t] = sum_k weights[t][k] * (ids[t][k] >= n_experts ? h[t] : y[t * top_k + k]) in slot order. */
 int mi_moe_combine_f32(const float* y, const float* h, int64_t ldh, const int32_t* ids, const float* weights,
                        int n_tokens, int top_k, int n_experts, int width, float* out, int64_t ldo, mi_stream stream);
@@ -718,6 +728,7 @@ int mi_moe_combine_f32(const float* y, const float* h, int64_t ldh, const int32_
 #define MI_ACT_GELU_TANH 2  /* 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))) */
 #define MI_ACT_GELU_ERF  3  /* 0.5 z (1 + erf(z / sqrt 2)) */
 #define MI_ACT_SIGMOID   4
+#define MI_ACT_SOFTCAP   5  /* alpha tanh(z / alpha): the epilogue's alpha is the cap (mi_gemm_any_act, no w2) */
 /* mi_gemm_any with an epilogue: v = x w^T + bias (bias may be NULL); w2 != NULL: y = alpha * act(v) * (x w2^T + bias2),
  * else y = alpha * act(v). */
 int mi_gemm_any_act(const float* x, int64_t ldx, const void* w, const void* w2, int w_dtype, const float* bias,
@@ -739,14 +750,15 @@ int mi_gemm_any_batched(const float* x, int64_t ldx, int64_t x_batch, const void
 #define MI_BIAS_NONE  2
 /* mi_swa_attention with the bias named and the value rows ldv elements apart: v_cache may be k_cache itself with
  * ldv = D when a token's value is the first Dv channels of its key row (latent attention: G = 1).  window >= the longest
- * sequence: plain causal attention.  workspace (may be NULL; workspace_elems floats): lets decode steps with few
+ * sequence: plain causal attention.  sink != NULL: every row's softmax denominator also holds exp(sink[h]), a logit per
+ * head without key or value (not scaled, counted once).  workspace (may be NULL; workspace_elems floats): lets decode steps with few
  * (row, kv head) units spread each unit's keys over several workgroups - rows * H * 2 k * (2 + Dv) floats allow k of
  * them, up to 16. */
 int mi_paged_attention_f32(const float* q, int64_t ldq, const void* k_cache, const void* v_cache, int64_t ldv,
                            int cache_dtype, const int32_t* block_tables, int table_cols, const int32_t* cu_q,
                            const int32_t* kv_lens, int n_seqs, int rows, int H, int G, int D, int Dv, int block_size,
                            int window, float scale, int bias_kind, const float* bias_p1, const float* bias_p2,
-                           const float* gate, int64_t ldg, float* out, int64_t ldo, float* workspace,
+                           const float* sink, const float* gate, int64_t ldg, float* out, int64_t ldo, float* workspace,
                            int64_t workspace_elems, mi_stream stream);
 /* res += mult * y (y may be NULL); w != NULL: out = res / sqrt(mean(res^2) + eps) * (w + shift) per row. */
 int mi_add_rmsnorm_f32(float* res, int64_t ldr, const float* y, int64_t ldy, float mult, const float* w, float shift,
@@ -768,11 +780,13 @@ int mi_mingru_scan(const float* proj, int64_t ld, int z_off, int x_off, int g_of
 int mi_kv_store_temp(float* proj, int64_t ld, int q_off, int k_off, int v_off, float temp_coef, int temp_every,
                      const int32_t* cu_q, const int32_t* kv_lens, int n_seqs, void* k_cache, void* v_cache, int cache_dtype,
                      const int32_t* slots, int rows, int H, int G, int D, int Dv, int block_size, mi_stream stream);
-/* Latent attention, per row: cache row [slot] = [rms(c) * norm_w | rot(r)] (c: C entries at c_off, r: the R behind
- * them); qx[row][h][C .. C + R) = rot(q_h[D .. D + R)) for every head (q heads of D + R entries at q_off).  rot turns
+/* Latent attention, per row: cache row [slot] = [rms(c) * norm_w | rot(r)] (c: C entries at c_off of proj, r: the R behind
+ * them); qx[row][h][C .. C + R) = rot(q_h[D .. D + R)) for every head (q heads of D + R entries at q_off of q's rows - q
+ * may be proj itself).  rot turns
  * the first rot_dims entries: pairs (i, i + rot_dims/2), angle pos * inv_freq[i] (a table of rot_dims/2 floats:
  * base^(-2 i / rot_dims)). */
-int mi_latent_prepare(const float* proj, int64_t ld, int q_off, int c_off, int H, int D, int R, int C, int rot_dims,
+int mi_latent_prepare(const float* proj, int64_t ld, const float* q, int64_t ldq, int q_off, int c_off, int H, int D,
+                      int R, int C, int rot_dims,
                       const float* inv_freq, const float* norm_w, float eps, const int32_t* cu_q, const int32_t* kv_lens,
                       int n_seqs, void* cache, int cache_dtype, const int32_t* slots, float* qx, int64_t ldqx, int rows,
                       mi_stream stream);
@@ -783,6 +797,29 @@ int mi_route_topk(const float* logits, int64_t ld, int n_tokens, int n_outputs, 
 int mi_moe_combine_shared(const float* y, const int32_t* ids, const float* weights, int n_tokens, int top_k, int width,
                           const float* shared, int64_t ld_shared, const float* shared_gate, int64_t ld_gate, float* out,
                           int64_t ldo, mi_stream stream);
+
+/* A gated sublayer output behind its own RMS norm, added to the residual stream: v = y * sigmoid(gate_pre) (gate_pre may
+ * be NULL: v = y); res += v / sqrt(mean(v^2) + eps) * w_post; w_next != NULL: out = res / sqrt(mean(res^2) + eps) * w_next
+ * (what the next sublayer reads). */
+int mi_gated_norm_add_f32(float* res, int64_t ldr, const float* y, int64_t ldy, const float* gate_pre, int64_t ldg,
+                          const float* w_post, float eps, const float* w_next, float* out, int64_t ldo, int rows, int width,
+                          mi_stream stream);
+#define MI_DECAY_HEAD   0  /* a_t = decay[h]: one constant per head */
+#define MI_DECAY_FORGET 1  /* a_t = f_t = lower + (1 - lower) sigmoid(z_t + f_bias) per key channel; k_t = 1 - f_t */
+/* Floats of state one sequence slot holds for mi_linear_attention (the kernel's own thread-order layout), or -1 when D
+ * is beyond the compiled kernels (D <= 256).  Host only. */
+int64_t mi_linear_attention_state_elems(int H, int D, int Dv);
+/* Linear attention with a decayed matrix state per head, fp32 state [slots][mi_linear_attention_state_elems]:
+ * S <- diag(a_t) S + k_t v_t^T;  o_t = S^T q_t.  proj rows hold q [H*D] at q_off, v [H*Dv] at v_off and at k_off either
+ * k [H*D] (MI_DECAY_HEAD) or the forget gate's pre-activation z [H*D] (MI_DECAY_FORGET: f_bias, lower [H*D]); q_act /
+ * k_act / v_act: MI_ACT_NONE or MI_ACT_SILU on the projections.  norm_w != NULL: the read-out is RMS-normed (eps inside
+ * the root) per head over Dv with norm_w [Dv] (norm_groups == H) or over all heads together with norm_w [H*Dv]
+ * (norm_groups == 1), then times sigmoid(gate_pre[row][..]) if gate_pre != NULL. */
+int mi_linear_attention(const float* proj, int64_t ld, int q_off, int k_off, int v_off, int q_act, int k_act, int v_act,
+                        int decay_kind, const float* decay, const float* f_bias, const float* lower, const float* gate_pre,
+                        int64_t ld_gate, const float* norm_w, int norm_groups, float* state, const int32_t* cu_q,
+                        const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int n_rows, int H, int D, int Dv,
+                        float eps, float* out, int64_t ldo, mi_stream stream);
 
 /* ---- host-side hashing (reference: engine/block_manager.py:38-44) --------- */
 /* xxh64 of `len` bytes with seed 0, optionally prefixed by the 8 little-endian

@@ -63,7 +63,7 @@ __device__ __forceinline__ float act_f(int act, float z) {
     case MI_ACT_GELU_TANH: return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
     case MI_ACT_GELU_ERF: return 0.5f * z * (1.f + erff(z * 0.7071067811865476f));
     case MI_ACT_SIGMOID: return 1.f / (1.f + expf(-z));
-    default: return z;
+    default: return z;  // (MI_ACT_SOFTCAP is finish()'s: it needs the cap)
   }
 }
 // what every kernel does to an accumulator (pair) before it stores it
@@ -74,7 +74,7 @@ __device__ __forceinline__ float finish(const GemmAnyArgs& a, int64_t yrow, int 
     if (a.bias2) v2 += a.bias2[n];
     v = act_f(a.act, v) * v2;
   } else {
-    v = act_f(a.act, v);
+    v = a.act == MI_ACT_SOFTCAP ? tanhf(v / a.alpha) : act_f(a.act, v);  // (times alpha below: alpha tanh(v / alpha))
   }
   v *= a.alpha;
   if (a.gate) v *= 1.f / (1.f + expf(-a.gate[yrow * a.ldgate + n]));
@@ -527,7 +527,7 @@ static int gemm_any_dispatch(const GemmAnyArgs& a, int w_dtype, int groups, int 
   return MI_EINVAL;
 }
 
-static bool act_ok(int act) { return act >= MI_ACT_NONE && act <= MI_ACT_SIGMOID; }
+static bool act_ok(int act) { return act >= MI_ACT_NONE && act <= MI_ACT_SOFTCAP; }
 
 extern "C" int mi_gemm_any(const float* x, int64_t ldx, const void* w, int w_dtype, float* y, int64_t ldy, int M, int N,
                            int K, float alpha, int exact, mi_stream stream) {
@@ -538,6 +538,7 @@ extern "C" int mi_gemm_any_act(const float* x, int64_t ldx, const void* w, const
                                const float* bias2, int act, float* y, int64_t ldy, int M, int N, int K, float alpha,
                                int exact, mi_stream stream) {
   if (!x || !w || !y || M < 0 || N < 0 || K < 1 || ldx < K || ldy < N || !act_ok(act) || (bias2 && !w2)) return MI_EINVAL;
+  if (act == MI_ACT_SOFTCAP && (w2 || !(alpha > 0.f))) return MI_EINVAL;
   GemmAnyArgs a{x, ldx, w, w2, y, ldy, M, N, K, alpha, nullptr, nullptr, nullptr, bias, bias2, act, nullptr, 0, 0, 0, 0};
   return gemm_any_dispatch(a, w_dtype, 1, M, exact ? 1 : 0, S(stream));
 }
@@ -564,7 +565,8 @@ extern "C" int mi_gemm_any_grouped_act(const float* x, int64_t ldx, const int32_
                                        int w_dtype, int act, const int32_t* group_offsets, int n_groups,
                                        int rows_per_group_max, float* y, int64_t ldy, const int32_t* y_rows, int N, int K,
                                        int exact, mi_stream stream) {
-  if (!x || !w || !y || !group_offsets || n_groups < 1 || rows_per_group_max < 0 || N < 0 || K < 1 || !act_ok(act))
+  if (!x || !w || !y || !group_offsets || n_groups < 1 || rows_per_group_max < 0 || N < 0 || K < 1 || !act_ok(act) ||
+      act == MI_ACT_SOFTCAP)
     return MI_EINVAL;
   if (n_groups > 65535) return MI_EUNSUPPORTED;
   GemmAnyArgs a{x, ldx, w, w2, y, ldy, rows_per_group_max, N, K, 1.0f, group_offsets, x_rows, y_rows, nullptr, nullptr,

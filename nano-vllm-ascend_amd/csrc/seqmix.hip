@@ -65,10 +65,12 @@ __device__ __forceinline__ int seq_of_row(const int32_t* cu_q, int n_seqs, int r
 
 template <typename TT>
 __global__ __launch_bounds__(256) void embedding_f32_kernel(const int64_t* __restrict__ ids, const TT* __restrict__ table,
-                                                            float* __restrict__ out, int width, int vocab) {
+                                                            float* __restrict__ out, int width, int vocab,
+                                                            float scale) {
   const int64_t id = ids[blockIdx.x];
   if (id < 0 || id >= vocab) return;
-  for (int c = threadIdx.x; c < width; c += 256) out[(int64_t)blockIdx.x * width + c] = ld_f<TT>(table + id * width + c);
+  for (int c = threadIdx.x; c < width; c += 256)
+    out[(int64_t)blockIdx.x * width + c] = ld_f<TT>(table + id * width + c) * scale;
 }
 
 // one workgroup per row; mean, then the mean of squared deviations (two passes over the row, which stays in L1)
@@ -139,11 +141,18 @@ __global__ __launch_bounds__(256) void swa_prepare_kernel(float* __restrict__ pr
 // Distance bias of a score, taken off it: kind MI_BIAS_SLOPE: 2^(-8 (h + 1) / H) * dist (p1 == nullptr) or p1[h] * dist;
 // MI_BIAS_LOG: p1[h] * ln(1 + p2[h] * dist); MI_BIAS_NONE: nothing.  ldv: elements between two tokens' value rows (Dv,
 // or the key row's length when the values are the leading channels of the key rows of the same cache).
+// sink != nullptr: the softmax's denominator also holds exp(sink[h]) - a learned logit per head that has no key and no
+// value, is not scaled and counts once per row.
 struct AttnBias {
   int kind;
   const float* p1;
   const float* p2;
+  const float* sink;
 };
+// the denominator of a finished row: its keys' sum l (relative to the running maximum m) plus the head's sink
+__device__ __forceinline__ float with_sink(const AttnBias& bias, int h, float m, float l) {
+  return bias.sink ? l + expf(bias.sink[h] - m) : l;
+}
 struct HeadBias {
   float a, b;
   bool log;
@@ -234,7 +243,7 @@ __global__ __launch_bounds__(256) void swa_attention_kernel(const float* __restr
     }
     __builtin_amdgcn_wave_barrier();
   }
-  const float inv = 1.f / l;
+  const float inv = 1.f / with_sink(bias, h, m, l);
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
     const int d = lane + 64 * i;
@@ -394,12 +403,13 @@ __global__ __launch_bounds__(256) void swa_attention_vec_kernel(const float* __r
           for (int e = 0; e < VEC; ++e) acc[0][e] = fmaf(part[w2 * (2 + Dv) + 2 + cg * VEC + e], f, acc[0][e]);
       }
       l[0] = lsum;
+      m[0] = mm;
     }
     if (kg == 0 && cg * VEC < Dv) {
 #pragma unroll
       for (int r = 0; r < RPW; ++r) {
         if (r >= nr) continue;
-        const float inv = 1.f / l[r];
+        const float inv = 1.f / with_sink(bias, h, m[r], l[r]);
         const int64_t row = first + r;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
@@ -583,7 +593,7 @@ __global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __
     if (qi < nr) {
       // the lane holds channels 16 dt + 4 kg + r of its query's output (PAIR: tile 2 dp + b holds the channels
       // 32 dp + 2 (4 kg + r) + b, i.e. the lane has the eight consecutive channels 32 dp + 8 kg .. + 7)
-      const float inv = 1.f / l;
+      const float inv = 1.f / with_sink(bias, h, m, l);
       const int64_t row = first + qi;
 #pragma unroll
       for (int dt = 0; dt < DVM; ++dt) {
@@ -808,7 +818,7 @@ __global__ __launch_bounds__(256) void paged_attention_heads_mfma_kernel(
     }
     return;
   }
-  const float inv = 1.f / l;
+  const float inv = 1.f / with_sink(bias, h0 + qi, mm, l);
   const int64_t obase = (int64_t)row * ldo + (int64_t)(h0 + qi) * Dv;
   const int64_t gbase = (int64_t)row * ldg + (int64_t)(h0 + qi) * Dv;
 #pragma unroll
@@ -830,6 +840,7 @@ __global__ __launch_bounds__(256) void paged_attention_heads_mfma_kernel(
 template <int NS>
 __global__ __launch_bounds__(256) void paged_attention_merge_kernel(const float* __restrict__ ws, int n_units, int H, int Dv,
                                                                     const float* __restrict__ gate, int64_t ldg,
+                                                                    const float* __restrict__ sink,
                                                                     float* __restrict__ out, int64_t ldo) {
   const int unit = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (unit >= n_units) return;
@@ -847,6 +858,7 @@ __global__ __launch_bounds__(256) void paged_attention_merge_kernel(const float*
     f[i] = m[i] == -INFINITY ? 0.f : expf(m[i] - mm);
     l = fmaf(p[i * stride + 1], f[i], l);
   }
+  if (sink) l += expf(sink[h] - mm);
   const float inv = 1.f / l;
   for (int d = lane; d < Dv; d += 64) {
     float v[NS];
@@ -864,15 +876,17 @@ __global__ __launch_bounds__(256) void paged_attention_merge_kernel(const float*
 // ---------------------------------------------------------------------------------------------------------------
 // short causal convolution with a carried tail
 // ---------------------------------------------------------------------------------------------------------------
-// y[r][c] = silu(sum_j w[c][j] * in[r - (taps - 1) + j]); inputs before the step's first row come from the sequence's
-// state slot (the last taps - 1 inputs, oldest first) - zeros when the sequence starts in this step.
-__global__ __launch_bounds__(256) void causal_conv_silu_kernel(const float* __restrict__ x, int64_t ldx,
+// y[r][c] = act(sum_j w[c][j] * in[r - (taps - 1) + j]) (+ in[r] when add_input); inputs before the step's first row
+// come from the sequence's state slot (the last taps - 1 inputs, oldest first) - zeros when the sequence starts in this
+// step.  silu: act = silu, else the identity.
+__global__ __launch_bounds__(256) void causal_conv_kernel(const float* __restrict__ x, int64_t ldx,
                                                                const float* __restrict__ w, int taps,
                                                                const float* __restrict__ state,
                                                                const int32_t* __restrict__ cu_q,
                                                                const int32_t* __restrict__ kv_lens,
                                                                const int32_t* __restrict__ slot_ids, int n_seqs, int C,
-                                                               float* __restrict__ y, int64_t ldy) {
+                                                               int silu, int add_input, float* __restrict__ y,
+                                                               int64_t ldy) {
   const int row = blockIdx.x;
   const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= C) return;
@@ -888,7 +902,9 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(const float* __re
     else v = start > 0 ? st[(int64_t)(taps - 1 + rr) * C + c] : 0.f;  // (a state written at position p holds inputs p-taps+1..p-1, zeros before 0)
     acc = fmaf(w[(int64_t)c * taps + j], v, acc);
   }
-  y[(int64_t)row * ldy + c] = acc / (1.f + expf(-acc));
+  if (silu) acc = acc / (1.f + expf(-acc));
+  if (add_input) acc += x[(int64_t)row * ldx + c];
+  y[(int64_t)row * ldy + c] = acc;
 }
 
 // the new tail: the last taps - 1 inputs of (old tail ++ this step's rows).  One thread per (sequence, channel) reads
@@ -1056,7 +1072,7 @@ __global__ __launch_bounds__(kDeltaThreads) void channel_delta_kernel(const floa
   for (int ii = 0; ii < DR; ++ii) slot[ii * kDeltaThreads + tid] = st[ii];
 }
 
-// out[row][h] <- out / rms(out over Dv) * norm_w * sigmoid(gate): one wave per (row, head), in place
+// out[row][h] <- out / rms(out over Dv) * norm_w (* sigmoid(gate) with a gate): one wave per (row, head), in place
 __global__ __launch_bounds__(256) void delta_finish_kernel(float* __restrict__ out, int64_t ldo,
                                                            const float* __restrict__ gate_pre, int64_t ld_gate,
                                                            const float* __restrict__ norm_w, int n_rows, int H, int Dv,
@@ -1070,7 +1086,7 @@ __global__ __launch_bounds__(256) void delta_finish_kernel(float* __restrict__ o
   for (int d = lane; d < Dv; d += 64) sq = fmaf(o[d], o[d], sq);
   const float rstd = 1.f / sqrtf(wave_sum(sq) / (float)Dv + eps);
   for (int d = lane; d < Dv; d += 64)
-    o[d] = o[d] * rstd * norm_w[d] * sigmoid_f(gate_pre[(int64_t)row * ld_gate + h * Dv + d]);
+    o[d] = o[d] * rstd * norm_w[d] * (gate_pre ? sigmoid_f(gate_pre[(int64_t)row * ld_gate + h * Dv + d]) : 1.f);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -1088,10 +1104,13 @@ __device__ __forceinline__ void wave_argmax(float& v, int& idx) {
   }
 }
 
+// score_kind: MI_ROUTE_SOFTMAX (scores = softmax over the outputs) or MI_ROUTE_SIGMOID (each output's own sigmoid);
+// group_kind: a group's value is its best choice score (MI_ROUTE_GROUP_MAX) or the sum of its two best
+// (MI_ROUTE_GROUP_TOP2; a group of one output: that output's score).
 __global__ __launch_bounds__(256) void route_grouped_kernel(const float* __restrict__ logits, int64_t ld,
                                                             const float* __restrict__ correction, int T, int n, int top_k,
-                                                            int n_groups, int keep, int32_t* __restrict__ ids,
-                                                            float* __restrict__ wts) {
+                                                            int n_groups, int keep, int score_kind, int group_kind,
+                                                            int32_t* __restrict__ ids, float* __restrict__ wts) {
   __shared__ float choice_s[4][512];
   __shared__ int kept_s[4][512];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -1110,12 +1129,18 @@ __global__ __launch_bounds__(256) void route_grouped_kernel(const float* __restr
   }
   mx = wave_max(mx);
   float sum = 0.f;
+  if (score_kind == MI_ROUTE_SOFTMAX) {
 #pragma unroll
-  for (int i = 0; i < EPL; ++i) {
-    sc[i] = lane + 64 * i < n ? expf(sc[i] - mx) : 0.f;
-    sum += sc[i];
+    for (int i = 0; i < EPL; ++i) {
+      sc[i] = lane + 64 * i < n ? expf(sc[i] - mx) : 0.f;
+      sum += sc[i];
+    }
+    sum = wave_sum(sum);
+  } else {
+    sum = 1.f;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) sc[i] = lane + 64 * i < n ? sigmoid_f(sc[i]) : 0.f;
   }
-  sum = wave_sum(sum);
 #pragma unroll
   for (int i = 0; i < EPL; ++i) {
     const int e = lane + 64 * i;
@@ -1133,7 +1158,13 @@ __global__ __launch_bounds__(256) void route_grouped_kernel(const float* __restr
     const int gi = lane + 64 * i;
     float gv = -INFINITY;
     if (gi < n_groups) {
-      for (int e = gi * per; e < (gi + 1) * per; ++e) gv = fmaxf(gv, choice_s[wave][e]);
+      float second = -INFINITY;
+      for (int e = gi * per; e < (gi + 1) * per; ++e) {
+        const float c = choice_s[wave][e];
+        if (c > gv) second = gv, gv = c;
+        else if (c > second) second = c;
+      }
+      if (group_kind == MI_ROUTE_GROUP_TOP2 && per > 1) gv += second;
       kept_s[wave][gi] = 0;
     }
     gsc[i] = gv;
@@ -1416,7 +1447,8 @@ __global__ __launch_bounds__(256) void kv_store_temp_kernel(float* __restrict__ 
 // pos * inv_freq[i] formed and turned into sine and cosine in fp32 (sincosf of the device library); inv_freq [dims / 2]
 // is the host's table of base^(-2 i / dims), rounded once from double.
 template <typename TC>
-__global__ __launch_bounds__(256) void latent_prepare_kernel(const float* __restrict__ proj, int64_t ld, int q_off,
+__global__ __launch_bounds__(256) void latent_prepare_kernel(const float* __restrict__ proj, int64_t ld,
+                                                             const float* __restrict__ q, int64_t ldq, int q_off,
                                                              int c_off, int H, int D, int R, int C, int dims,
                                                              const float* __restrict__ inv_freq,
                                                              const float* __restrict__ norm_w, float eps,
@@ -1440,7 +1472,7 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(const float* __rest
   // unit u = 0: the shared key part; u = 1 + h: query head h
   for (int i = threadIdx.x; i < (H + 1) * R; i += 256) {
     const int u = i / R, e = i % R;
-    const float* src = u == 0 ? r + c_off + C : r + q_off + (int64_t)(u - 1) * (D + R) + D;
+    const float* src = u == 0 ? r + c_off + C : q + (int64_t)row * ldq + q_off + (int64_t)(u - 1) * (D + R) + D;
     float v = src[e];
     if (e < dims) {
       const int f = e < half ? e : e - half;
@@ -1522,20 +1554,177 @@ __global__ __launch_bounds__(256) void moe_combine_shared_kernel(const float* __
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------------------------
+// gated sublayer output behind its own norm, added to the residual: res += rms(y * sigmoid(gate)) * w_post
+// ---------------------------------------------------------------------------------------------------------------
+// One workgroup per row.  v = y * sigmoid(gate_pre) (gate_pre may be nullptr: v = y); res += v / sqrt(mean(v^2) + eps) *
+// w_post; w_next != nullptr: out = res / sqrt(mean(res^2) + eps) * w_next - what the next sublayer reads.  A thread keeps
+// its (up to eight) gated values in registers between the two passes; wider rows recompute them.
+__global__ __launch_bounds__(256) void gated_norm_add_f32_kernel(float* __restrict__ res, int64_t ldr,
+                                                                 const float* __restrict__ y, int64_t ldy,
+                                                                 const float* __restrict__ gate_pre, int64_t ldg,
+                                                                 const float* __restrict__ w_post, float eps,
+                                                                 const float* __restrict__ w_next,
+                                                                 float* __restrict__ out, int64_t ldo, int width) {
+  __shared__ float red[4];
+  constexpr int KEEP = 8;
+  float* r = res + (int64_t)blockIdx.x * ldr;
+  const float* yr = y + (int64_t)blockIdx.x * ldy;
+  const float* gr = gate_pre ? gate_pre + (int64_t)blockIdx.x * ldg : nullptr;
+  float kept[KEEP];
+  float sq = 0.f;
+  int i = 0;
+  for (int c = threadIdx.x; c < width; c += 256, ++i) {
+    float v = yr[c];
+    if (gr) v *= sigmoid_f(gr[c]);
+    if (i < KEEP) kept[i] = v;
+    sq = fmaf(v, v, sq);
+  }
+  const float rstd = 1.f / sqrtf(block_sum256(sq, red) / (float)width + eps);
+  float sq2 = 0.f;
+  i = 0;
+  for (int c = threadIdx.x; c < width; c += 256, ++i) {
+    float v;
+    if (i < KEEP) v = kept[i];
+    else {
+      v = yr[c];
+      if (gr) v *= sigmoid_f(gr[c]);
+    }
+    const float x = fmaf(v * rstd, w_post[c], r[c]);
+    r[c] = x;
+    if (i < KEEP) kept[i] = x;
+    sq2 = fmaf(x, x, sq2);
+  }
+  if (!w_next) return;
+  const float rstd2 = 1.f / sqrtf(block_sum256(sq2, red) / (float)width + eps);
+  float* o = out + (int64_t)blockIdx.x * ldo;
+  i = 0;
+  for (int c = threadIdx.x; c < width; c += 256, ++i) o[c] = (i < KEEP ? kept[i] : r[c]) * rstd2 * w_next[c];
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// linear attention with a decayed matrix state: S <- diag(a_t) S + k_t v_t^T,  o_t = S^T q_t
+// ---------------------------------------------------------------------------------------------------------------
+// Two kinds of decay (DECAY):
+//   MI_DECAY_HEAD    a_t = decay[h] for every key channel of head h and every row; q, k, v = act(projection)
+//   MI_DECAY_FORGET  a_t = f_t = lower + (1 - lower) * sigmoid(z_t + f_bias) per key channel (z at k_off), and what is
+//                    written is k_t = 1 - f_t: the forget gate also decides how much of v_t enters
+// The walk is channel_delta_kernel's: a workgroup = 32 value columns of one (sequence, head); a column is held by a quad
+// of lanes, lane r of it keeping the key channels (4 jj + r) * 4 + e in registers for the whole walk over the step's
+// rows; the rows' vectors of 16 rows at a time go through LDS, loaded one batch ahead as raw projections and turned into
+// q / k / a (activations, gate) on their way into LDS - no separate preparation launch; sums over the key channels end
+// in two DPP steps inside the quad.  The state lives in memory in thread order ([slot][head][column block][DR][128]).
+template <int DR, int DECAY>
+__global__ __launch_bounds__(kDeltaThreads) void linear_attention_kernel(
+    const float* __restrict__ proj, int64_t ld, int q_off, int k_off, int v_off, int q_act, int k_act, int v_act,
+    const float* __restrict__ decay, const float* __restrict__ f_bias, const float* __restrict__ lower,
+    float* __restrict__ state, const int32_t* __restrict__ cu_q, const int32_t* __restrict__ kv_lens,
+    const int32_t* __restrict__ slot_ids, int H, int D, int Dv, float* __restrict__ out, int64_t ldo) {
+  constexpr int DP = 4 * DR;  // padded key channels
+  constexpr bool FORGET = DECAY == MI_DECAY_FORGET;
+  __shared__ __attribute__((aligned(16))) float qs[kDeltaRows][DP];
+  __shared__ __attribute__((aligned(16))) float ks[kDeltaRows][DP];
+  __shared__ __attribute__((aligned(16))) float gs[FORGET ? kDeltaRows : 1][DP];
+  __shared__ float vs[kDeltaRows][kDeltaCols];
+  const int s = blockIdx.x, h = blockIdx.y, cb = blockIdx.z;
+  const int tid = threadIdx.x, r = tid & 3, col = tid >> 2;
+  const int c = cb * kDeltaCols + col;
+  const int r0 = cu_q[s], n = cu_q[s + 1] - r0;
+  if (n == 0) return;
+  const int start = kv_lens[s] - n;
+  float* slot = state + (((int64_t)slot_ids[s] * H + h) * gridDim.z + cb) * DR * kDeltaThreads;
+  float st[DR];
+#pragma unroll
+  for (int ii = 0; ii < DR; ++ii) st[ii] = start > 0 ? slot[ii * kDeltaThreads + tid] : 0.f;
+  const float head_decay = FORGET ? 0.f : decay[h];
+  // staging: 8 lanes per row copy the row's vectors (zeros beyond D and beyond the step's rows)
+  const int pt = tid >> 3, ps = tid & 7;
+  constexpr int PE = DP / 8;
+  float rq[PE], rk[PE], rv[kDeltaCols / 8];
+  auto fetch = [&](int c0) {
+    const bool live = c0 + pt < n;
+    const int64_t row = r0 + (live ? c0 + pt : 0);
+    const float* p = proj + row * ld;
+#pragma unroll
+    for (int m = 0; m < PE; ++m) {
+      const int i = ps + 8 * m;
+      const bool ok = live && i < D;
+      rq[m] = ok ? p[q_off + h * D + i] : 0.f;
+      rk[m] = ok ? p[k_off + h * D + i] : 0.f;
+    }
+#pragma unroll
+    for (int m = 0; m < kDeltaCols / 8; ++m) {
+      const int cc = cb * kDeltaCols + ps + 8 * m;
+      rv[m] = (live && cc < Dv) ? p[v_off + h * Dv + cc] : 0.f;
+    }
+  };
+  auto act = [](int kind, float z) { return kind == MI_ACT_SILU ? z / (1.f + expf(-z)) : z; };
+  fetch(0);
+  for (int c0 = 0; c0 < n; c0 += kDeltaRows) {
+    __syncthreads();  // the previous rows' vectors have been consumed
+    const bool live = c0 + pt < n;
+#pragma unroll
+    for (int m = 0; m < PE; ++m) {
+      const int i = ps + 8 * m;
+      const bool ok = live && i < D;
+      qs[pt][i] = ok ? act(q_act, rq[m]) : 0.f;
+      if constexpr (FORGET) {
+        const float lo = i < D ? lower[h * D + i] : 0.f, fb = i < D ? f_bias[h * D + i] : 0.f;  // (cached: every batch)
+        const float f = lo + (1.f - lo) * sigmoid_f(rk[m] + fb);
+        gs[pt][i] = ok ? f : 0.f;
+        ks[pt][i] = ok ? 1.f - f : 0.f;
+      } else {
+        ks[pt][i] = ok ? act(k_act, rk[m]) : 0.f;
+      }
+    }
+#pragma unroll
+    for (int m = 0; m < kDeltaCols / 8; ++m) vs[pt][ps + 8 * m] = act(v_act, rv[m]);
+    __syncthreads();
+    if (c0 + kDeltaRows < n) fetch(c0 + kDeltaRows);
+    const int nt = min(kDeltaRows, n - c0);
+    for (int t = 0; t < nt; ++t) {
+      const float4* k4 = reinterpret_cast<const float4*>(ks[t]);
+      const float4* q4 = reinterpret_cast<const float4*>(qs[t]);
+      const float4* g4 = reinterpret_cast<const float4*>(gs[FORGET ? t : 0]);
+      const float v = vs[t][col];
+      float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+#pragma unroll
+      for (int jj = 0; jj < DR / 4; ++jj) {
+        const float4 kv = k4[jj * 4 + r], qv = q4[jj * 4 + r];
+        float4 gv{head_decay, head_decay, head_decay, head_decay};
+        if constexpr (FORGET) gv = g4[jj * 4 + r];
+        st[jj * 4 + 0] = fmaf(gv.x, st[jj * 4 + 0], kv.x * v);
+        st[jj * 4 + 1] = fmaf(gv.y, st[jj * 4 + 1], kv.y * v);
+        st[jj * 4 + 2] = fmaf(gv.z, st[jj * 4 + 2], kv.z * v);
+        st[jj * 4 + 3] = fmaf(gv.w, st[jj * 4 + 3], kv.w * v);
+        o0 = fmaf(st[jj * 4 + 0], qv.x, o0);
+        o1 = fmaf(st[jj * 4 + 1], qv.y, o1);
+        o2 = fmaf(st[jj * 4 + 2], qv.z, o2);
+        o3 = fmaf(st[jj * 4 + 3], qv.w, o3);
+      }
+      const float o = xor_sum<2>(xor_sum<1>((o0 + o1) + (o2 + o3)));
+      if (r == 0 && c < Dv) out[(int64_t)(r0 + c0 + t) * ldo + h * Dv + c] = o;
+    }
+  }
+#pragma unroll
+  for (int ii = 0; ii < DR; ++ii) slot[ii * kDeltaThreads + tid] = st[ii];
+}
+
 }  // namespace mi
 
 using namespace mi;
 
 extern "C" int mi_embedding_f32(const int64_t* ids, const void* table, int table_dtype, float* out, int n, int width,
-                                int vocab, mi_stream stream) {
+                                int vocab, float scale, mi_stream stream) {
   if (!ids || !table || !out || n < 0 || width < 1) return MI_EINVAL;
   if (n == 0) return MI_OK;
   if (table_dtype == MI_DTYPE_BF16)
     hipLaunchKernelGGL((embedding_f32_kernel<uint16_t>), dim3(n), dim3(256), 0, S(stream), ids,
-                       static_cast<const uint16_t*>(table), out, width, vocab);
+                       static_cast<const uint16_t*>(table), out, width, vocab, scale);
   else if (table_dtype == MI_DTYPE_F32)
     hipLaunchKernelGGL((embedding_f32_kernel<float>), dim3(n), dim3(256), 0, S(stream), ids,
-                       static_cast<const float*>(table), out, width, vocab);
+                       static_cast<const float*>(table), out, width, vocab, scale);
   else return MI_EINVAL;
   return check_launch();
 }
@@ -1617,7 +1806,7 @@ static int launch_swa(const float* q, int64_t ldq, const void* kc, const void* v
       if (n_split == 1) return MI_OK;
 #define MI_MERGE(NS)                                                                                                  \
   hipLaunchKernelGGL((paged_attention_merge_kernel<NS>), dim3((rows * H + 3) / 4), dim3(256), 0, st, ws, rows * H, H, Dv, \
-                     gate, ldg, out, ldo)
+                     gate, ldg, bias.sink, out, ldo)
       if (n_split == 2) MI_MERGE(2);
       else if (n_split == 4) MI_MERGE(4);
       else if (n_split == 8) MI_MERGE(8);
@@ -1663,23 +1852,24 @@ extern "C" int mi_swa_attention(const float* q, int64_t ldq, const void* k_cache
                                 int n_seqs, int rows, int H, int G, int D, int Dv, int block_size, int window,
                                 float scale, const float* gate, int64_t ldg, float* out, int64_t ldo, mi_stream stream) {
   return mi_paged_attention_f32(q, ldq, k_cache, v_cache, Dv, cache_dtype, block_tables, table_cols, cu_q, kv_lens, n_seqs,
-                                rows, H, G, D, Dv, block_size, window, scale, MI_BIAS_SLOPE, nullptr, nullptr, gate, ldg,
-                                out, ldo, nullptr, 0, stream);
+                                rows, H, G, D, Dv, block_size, window, scale, MI_BIAS_SLOPE, nullptr, nullptr, nullptr, gate,
+                                ldg, out, ldo, nullptr, 0, stream);
 }
 
 extern "C" int mi_paged_attention_f32(const float* q, int64_t ldq, const void* k_cache, const void* v_cache, int64_t ldv,
                                       int cache_dtype, const int32_t* block_tables, int table_cols, const int32_t* cu_q,
                                       const int32_t* kv_lens, int n_seqs, int rows, int H, int G, int D, int Dv,
                                       int block_size, int window, float scale, int bias_kind, const float* bias_p1,
-                                      const float* bias_p2, const float* gate, int64_t ldg, float* out, int64_t ldo,
-                                      float* workspace, int64_t workspace_elems, mi_stream stream) {
+                                      const float* bias_p2, const float* sink, const float* gate, int64_t ldg,
+                                      float* out, int64_t ldo, float* workspace, int64_t workspace_elems,
+                                      mi_stream stream) {
   if (!q || !k_cache || !v_cache || !block_tables || !cu_q || !kv_lens || !out || rows < 0 || n_seqs < 1) return MI_EINVAL;
   if (H < 1 || G < 1 || H % G || D < 1 || Dv < 1 || block_size < 1 || window < 1 || table_cols < 1 || ldv < Dv) return MI_EINVAL;
   if (bias_kind != MI_BIAS_SLOPE && bias_kind != MI_BIAS_LOG && bias_kind != MI_BIAS_NONE) return MI_EINVAL;
   if (bias_kind == MI_BIAS_LOG && (!bias_p1 || !bias_p2)) return MI_EINVAL;
   if (Dv > 512 || D > 4096) return MI_EUNSUPPORTED;
   if (rows == 0) return MI_OK;
-  const AttnBias bias{bias_kind, bias_p1, bias_p2};
+  const AttnBias bias{bias_kind, bias_p1, bias_p2, sink};
   if (cache_dtype == MI_DTYPE_BF16)
     return launch_swa<uint16_t>(q, ldq, k_cache, v_cache, block_tables, table_cols, cu_q, kv_lens, n_seqs, rows, H, G, D,
                                 Dv, block_size, window, scale, bias, ldv, gate, ldg, out, ldo, workspace, workspace_elems,
@@ -1691,15 +1881,21 @@ extern "C" int mi_paged_attention_f32(const float* q, int64_t ldq, const void* k
   return MI_EINVAL;
 }
 
-extern "C" int mi_causal_conv_silu(const float* x, int64_t ldx, const float* w, int taps, const float* state,
-                                   const int32_t* cu_q, const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs,
-                                   int rows, int channels, float* y, int64_t ldy, mi_stream stream) {
+extern "C" int mi_causal_conv(const float* x, int64_t ldx, const float* w, int taps, const float* state,
+                              const int32_t* cu_q, const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int rows,
+                              int channels, int silu, int add_input, float* y, int64_t ldy, mi_stream stream) {
   if (!x || !w || !state || !cu_q || !kv_lens || !slot_ids || !y || rows < 0 || n_seqs < 1 || channels < 1) return MI_EINVAL;
   if (taps < 1 || taps > 17) return MI_EUNSUPPORTED;
   if (rows == 0) return MI_OK;
-  hipLaunchKernelGGL(causal_conv_silu_kernel, dim3(rows, (channels + 255) / 256), dim3(256), 0, S(stream), x, ldx, w,
-                     taps, state, cu_q, kv_lens, slot_ids, n_seqs, channels, y, ldy);
+  hipLaunchKernelGGL(causal_conv_kernel, dim3(rows, (channels + 255) / 256), dim3(256), 0, S(stream), x, ldx, w, taps,
+                     state, cu_q, kv_lens, slot_ids, n_seqs, channels, silu, add_input, y, ldy);
   return check_launch();
+}
+
+extern "C" int mi_causal_conv_silu(const float* x, int64_t ldx, const float* w, int taps, const float* state,
+                                   const int32_t* cu_q, const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs,
+                                   int rows, int channels, float* y, int64_t ldy, mi_stream stream) {
+  return mi_causal_conv(x, ldx, w, taps, state, cu_q, kv_lens, slot_ids, n_seqs, rows, channels, 1, 0, y, ldy, stream);
 }
 
 extern "C" int mi_causal_conv_state(const float* x, int64_t ldx, int taps, float* state, const int32_t* cu_q,
@@ -1757,14 +1953,18 @@ extern "C" int mi_channel_delta(const float* qkv, int64_t ld, int q_off, int k_o
 }
 
 extern "C" int mi_route_grouped(const float* logits, int64_t ld, const float* correction, int n_tokens, int n_outputs,
-                                int top_k, int n_groups, int keep, int32_t* ids, float* weights, mi_stream stream) {
+                                int top_k, int n_groups, int keep, int score_kind, int group_kind, int32_t* ids,
+                                float* weights, mi_stream stream) {
   if (!logits || !correction || !ids || !weights || n_tokens < 0) return MI_EINVAL;
+  if ((score_kind != MI_ROUTE_SOFTMAX && score_kind != MI_ROUTE_SIGMOID) ||
+      (group_kind != MI_ROUTE_GROUP_MAX && group_kind != MI_ROUTE_GROUP_TOP2))
+    return MI_EINVAL;
   if (n_outputs < 1 || n_outputs > 512 || n_groups < 1 || n_outputs % n_groups || keep < 1 || keep > n_groups ||
       top_k < 1 || top_k > keep * (n_outputs / n_groups))
     return MI_EUNSUPPORTED;
   if (n_tokens == 0) return MI_OK;
   hipLaunchKernelGGL(route_grouped_kernel, dim3((n_tokens + 3) / 4), dim3(256), 0, S(stream), logits, ld, correction,
-                     n_tokens, n_outputs, top_k, n_groups, keep, ids, weights);
+                     n_tokens, n_outputs, top_k, n_groups, keep, score_kind, group_kind, ids, weights);
   return check_launch();
 }
 
@@ -1849,22 +2049,22 @@ extern "C" int mi_kv_store_temp(float* proj, int64_t ld, int q_off, int k_off, i
   return check_launch();
 }
 
-extern "C" int mi_latent_prepare(const float* proj, int64_t ld, int q_off, int c_off, int H, int D, int R, int C,
-                                 int rot_dims, const float* inv_freq, const float* norm_w, float eps, const int32_t* cu_q,
+extern "C" int mi_latent_prepare(const float* proj, int64_t ld, const float* q, int64_t ldq, int q_off, int c_off, int H,
+                                 int D, int R, int C, int rot_dims, const float* inv_freq, const float* norm_w, float eps, const int32_t* cu_q,
                                  const int32_t* kv_lens, int n_seqs, void* cache, int cache_dtype, const int32_t* slots,
                                  float* qx, int64_t ldqx, int rows, mi_stream stream) {
-  if (!proj || !norm_w || !cu_q || !kv_lens || !cache || !slots || !qx || rows < 0 || n_seqs < 1) return MI_EINVAL;
+  if (!proj || !q || !norm_w || !cu_q || !kv_lens || !cache || !slots || !qx || rows < 0 || n_seqs < 1) return MI_EINVAL;
   if (H < 1 || D < 0 || R < 0 || C < 1 || rot_dims < 0 || rot_dims > R || rot_dims % 2 || ldqx < (int64_t)H * (C + R))
     return MI_EINVAL;
   if (rot_dims > 0 && !inv_freq) return MI_EINVAL;
   if (rows == 0) return MI_OK;
   if (cache_dtype == MI_DTYPE_BF16)
-    hipLaunchKernelGGL((latent_prepare_kernel<uint16_t>), dim3(rows), dim3(256), 0, S(stream), proj, ld, q_off, c_off, H, D,
-                       R, C, rot_dims, inv_freq, norm_w, eps, cu_q, kv_lens, n_seqs, static_cast<uint16_t*>(cache), slots,
+    hipLaunchKernelGGL((latent_prepare_kernel<uint16_t>), dim3(rows), dim3(256), 0, S(stream), proj, ld, q, ldq, q_off, c_off,
+                       H, D, R, C, rot_dims, inv_freq, norm_w, eps, cu_q, kv_lens, n_seqs, static_cast<uint16_t*>(cache), slots,
                        qx, ldqx);
   else if (cache_dtype == MI_DTYPE_F32)
-    hipLaunchKernelGGL((latent_prepare_kernel<float>), dim3(rows), dim3(256), 0, S(stream), proj, ld, q_off, c_off, H, D, R,
-                       C, rot_dims, inv_freq, norm_w, eps, cu_q, kv_lens, n_seqs, static_cast<float*>(cache), slots, qx,
+    hipLaunchKernelGGL((latent_prepare_kernel<float>), dim3(rows), dim3(256), 0, S(stream), proj, ld, q, ldq, q_off, c_off, H,
+                       D, R, C, rot_dims, inv_freq, norm_w, eps, cu_q, kv_lens, n_seqs, static_cast<float*>(cache), slots, qx,
                        ldqx);
   else return MI_EINVAL;
   return check_launch();
@@ -1887,5 +2087,61 @@ extern "C" int mi_moe_combine_shared(const float* y, const int32_t* ids, const f
   if (n_tokens == 0) return MI_OK;
   hipLaunchKernelGGL(moe_combine_shared_kernel, dim3(n_tokens), dim3(256), 0, S(stream), y, ids, weights, top_k, width,
                      shared, ld_shared, shared_gate, ld_gate, out, ldo);
+  return check_launch();
+}
+
+extern "C" int mi_gated_norm_add_f32(float* res, int64_t ldr, const float* y, int64_t ldy, const float* gate_pre,
+                                     int64_t ldg, const float* w_post, float eps, const float* w_next, float* out,
+                                     int64_t ldo, int rows, int width, mi_stream stream) {
+  if (!res || !y || !w_post || rows < 0 || width < 1 || (w_next && !out)) return MI_EINVAL;
+  if (rows == 0) return MI_OK;
+  hipLaunchKernelGGL(gated_norm_add_f32_kernel, dim3(rows), dim3(256), 0, S(stream), res, ldr, y, ldy, gate_pre, ldg,
+                     w_post, eps, w_next, out, ldo, width);
+  return check_launch();
+}
+
+extern "C" int64_t mi_linear_attention_state_elems(int H, int D, int Dv) {
+  const int dr = delta_dr(D);
+  if (!dr) return -1;
+  return (int64_t)H * ((Dv + kDeltaCols - 1) / kDeltaCols) * dr * kDeltaThreads;
+}
+
+extern "C" int mi_linear_attention(const float* proj, int64_t ld, int q_off, int k_off, int v_off, int q_act, int k_act,
+                                   int v_act, int decay_kind, const float* decay, const float* f_bias, const float* lower,
+                                   const float* gate_pre, int64_t ld_gate, const float* norm_w, int norm_groups,
+                                   float* state, const int32_t* cu_q, const int32_t* kv_lens, const int32_t* slot_ids,
+                                   int n_seqs, int n_rows, int H, int D, int Dv, float eps, float* out, int64_t ldo,
+                                   mi_stream stream) {
+  if (!proj || !state || !cu_q || !kv_lens || !slot_ids || !out || n_rows < 0 || n_seqs < 1) return MI_EINVAL;
+  if (H < 1 || D < 1 || Dv < 1 || ldo < (int64_t)H * Dv) return MI_EINVAL;
+  if (decay_kind == MI_DECAY_HEAD ? !decay : decay_kind == MI_DECAY_FORGET ? (!f_bias || !lower) : true) return MI_EINVAL;
+  if (norm_w && norm_groups != 1 && norm_groups != H) return MI_EINVAL;
+  for (int a : {q_act, k_act, v_act})
+    if (a != MI_ACT_NONE && a != MI_ACT_SILU) return MI_EUNSUPPORTED;
+  const int dr = delta_dr(D);
+  if (!dr || H > 65535) return MI_EUNSUPPORTED;
+  if (n_rows == 0) return MI_OK;
+  const dim3 grid(n_seqs, H, (Dv + kDeltaCols - 1) / kDeltaCols);
+#define MI_LINATTN(DR, KIND)                                                                                          \
+  hipLaunchKernelGGL((linear_attention_kernel<DR, KIND>), grid, dim3(kDeltaThreads), 0, S(stream), proj, ld, q_off,  \
+                     k_off, v_off, q_act, k_act, v_act, decay, f_bias, lower, state, cu_q, kv_lens, slot_ids, H, D, Dv, \
+                     out, ldo)
+  if (decay_kind == MI_DECAY_HEAD) {
+    if (dr == 16) MI_LINATTN(16, MI_DECAY_HEAD);
+    else if (dr == 32) MI_LINATTN(32, MI_DECAY_HEAD);
+    else MI_LINATTN(64, MI_DECAY_HEAD);
+  } else {
+    if (dr == 16) MI_LINATTN(16, MI_DECAY_FORGET);
+    else if (dr == 32) MI_LINATTN(32, MI_DECAY_FORGET);
+    else MI_LINATTN(64, MI_DECAY_FORGET);
+  }
+#undef MI_LINATTN
+  if (check_launch() != MI_OK) return MI_ELAUNCH;
+  if (!norm_w) return MI_OK;
+  // the read-out's norm: over each head's value channels (norm_groups == H, weight [Dv]) or over all heads' channels
+  // together (norm_groups == 1, weight [H * Dv]); then the sigmoid gate, if any
+  const int groups = norm_groups, gw = norm_groups == 1 ? H * Dv : Dv;
+  hipLaunchKernelGGL(delta_finish_kernel, dim3((n_rows * groups + 3) / 4), dim3(256), 0, S(stream), out, ldo, gate_pre,
+                     ld_gate, norm_w, n_rows, groups, gw, eps);
   return check_launch();
 }

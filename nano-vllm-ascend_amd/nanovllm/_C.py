@@ -25,7 +25,10 @@ LIB_PATH = os.environ.get(
 MI_OK = 0
 MI_EUNSUPPORTED = -2
 DTYPE_BF16, DTYPE_F32 = 0, 1
-ACT_NONE, ACT_SILU, ACT_GELU_TANH, ACT_GELU_ERF, ACT_SIGMOID = range(5)   # MI_ACT_*
+ACT_NONE, ACT_SILU, ACT_GELU_TANH, ACT_GELU_ERF, ACT_SIGMOID, ACT_SOFTCAP = range(6)   # MI_ACT_*
+ROUTE_SOFTMAX, ROUTE_SIGMOID = range(2)                                   # MI_ROUTE_*
+ROUTE_GROUP_MAX, ROUTE_GROUP_TOP2 = range(2)                              # MI_ROUTE_GROUP_*
+DECAY_HEAD, DECAY_FORGET = range(2)                                       # MI_DECAY_*
 BIAS_SLOPE, BIAS_LOG, BIAS_NONE = range(3)                                # MI_BIAS_*
 HEAD_DIM = 128
 KV_TILE_TOKENS = 16
@@ -169,19 +172,20 @@ _SIGNATURES = {
     "mi_gemm_any": (c_int, [_p, c_int64, _p, c_int, _p, c_int64, c_int, c_int, c_int, c_float, c_int, _p]),
     "mi_gemm_any_grouped": (c_int, [_p, c_int64, _p, _p, _p, c_int, _p, c_int, c_int, _p, c_int64, _p, c_int, c_int,
                                     c_int, _p]),
-    "mi_embedding_f32": (c_int, [_p, _p, c_int, _p, c_int, c_int, c_int, _p]),
+    "mi_embedding_f32": (c_int, [_p, _p, c_int, _p, c_int, c_int, c_int, c_float, _p]),
     "mi_layernorm_f32": (c_int, [_p, c_int64, _p, _p, _p, c_int64, c_int, c_int, c_float, c_int, _p]),
     "mi_swa_prepare": (c_int, [_p, c_int64, c_int, c_int, c_int, _p, _p, c_float, _p, c_int64, _p, _p, _p, c_int, _p,
                                c_int, c_int, c_int, c_int, c_int, c_int, _p]),
     "mi_swa_attention": (c_int, [_p, c_int64, _p, _p, c_int, _p, c_int, _p, _p, c_int, c_int, c_int, c_int, c_int,
                                  c_int, c_int, c_int, c_float, _p, c_int64, _p, c_int64, _p]),
     "mi_causal_conv_silu": (c_int, [_p, c_int64, _p, c_int, _p, _p, _p, _p, c_int, c_int, c_int, _p, c_int64, _p]),
+    "mi_causal_conv": (c_int, [_p, c_int64, _p, c_int, _p, _p, _p, _p, c_int, c_int, c_int, c_int, c_int, _p, c_int64, _p]),
     "mi_causal_conv_state": (c_int, [_p, c_int64, c_int, _p, _p, _p, _p, c_int, c_int, _p]),
     "mi_channel_delta_state_elems": (c_int64, [c_int, c_int, c_int]),
     "mi_channel_delta_workspace_elems": (c_int64, [c_int, c_int, c_int, c_int]),
     "mi_channel_delta": (c_int, [_p, c_int64, c_int, c_int, c_int, _p, c_int64, _p, c_int64, _p, _p, _p, c_int64, _p,
                                  _p, _p, _p, _p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _p, _p, c_int64, _p]),
-    "mi_route_grouped": (c_int, [_p, c_int64, _p, c_int, c_int, c_int, c_int, c_int, _p, _p, _p]),
+    "mi_route_grouped": (c_int, [_p, c_int64, _p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _p, _p, _p]),
     "mi_moe_combine_f32": (c_int, [_p, _p, c_int64, _p, _p, c_int, c_int, c_int, c_int, _p, c_int64, _p]),
     "mi_gemm_any_act": (c_int, [_p, c_int64, _p, _p, c_int, _p, _p, c_int, _p, c_int64, c_int, c_int, c_int, c_float,
                                 c_int, _p]),
@@ -190,7 +194,8 @@ _SIGNATURES = {
     "mi_gemm_any_batched": (c_int, [_p, c_int64, c_int64, _p, c_int, _p, c_int64, c_int64, _p, c_int64, c_int64, c_int,
                                     c_int, c_int, c_int, c_int, _p]),
     "mi_paged_attention_f32": (c_int, [_p, c_int64, _p, _p, c_int64, c_int, _p, c_int, _p, _p, c_int, c_int, c_int, c_int,
-                                       c_int, c_int, c_int, c_int, c_float, c_int, _p, _p, _p, c_int64, _p, c_int64, _p, c_int64, _p]),
+                                       c_int, c_int, c_int, c_int, c_float, c_int, _p, _p, _p, _p, c_int64, _p, c_int64, _p, c_int64,
+                                       _p]),
     "mi_add_rmsnorm_f32": (c_int, [_p, c_int64, _p, c_int64, c_float, _p, c_float, c_float, _p, c_int64, c_int, c_int, _p]),
     "mi_depth_mix_f32": (c_int, [_p, c_int64, c_int, _p, _p, c_int64, c_float, _p, c_float, c_float, _p, c_int64, c_int,
                                  c_int, _p]),
@@ -199,10 +204,14 @@ _SIGNATURES = {
                                c_int64, _p]),
     "mi_kv_store_temp": (c_int, [_p, c_int64, c_int, c_int, c_int, c_float, c_int, _p, _p, c_int, _p, _p, c_int, _p, c_int,
                                  c_int, c_int, c_int, c_int, c_int, _p]),
-    "mi_latent_prepare": (c_int, [_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _p, _p, c_float, _p,
+    "mi_latent_prepare": (c_int, [_p, c_int64, _p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _p, _p, c_float, _p,
                                   _p, c_int, _p, c_int, _p, _p, c_int64, c_int, _p]),
     "mi_route_topk": (c_int, [_p, c_int64, c_int, c_int, c_int, _p, _p, _p]),
     "mi_moe_combine_shared": (c_int, [_p, _p, _p, c_int, c_int, c_int, _p, c_int64, _p, c_int64, _p, c_int64, _p]),
+    "mi_gated_norm_add_f32": (c_int, [_p, c_int64, _p, c_int64, _p, c_int64, _p, c_float, _p, _p, c_int64, c_int, c_int, _p]),
+    "mi_linear_attention_state_elems": (c_int64, [c_int, c_int, c_int]),
+    "mi_linear_attention": (c_int, [_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _p, _p, _p, _p, c_int64,
+                                    _p, c_int, _p, _p, _p, _p, c_int, c_int, c_int, c_int, c_int, c_float, _p, c_int64, _p]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

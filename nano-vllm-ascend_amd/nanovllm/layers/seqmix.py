@@ -20,6 +20,12 @@ configuration:
   GatedDenseMLP             W_d (act(W_g h + b) * (W_u h + b)) + b
   SharedSparseMLP           top-k experts of the plain form W_d act(W_u h), softmax over the chosen logits, plus a shared
                             expert behind a per-token sigmoid gate
+  InputConvolution          what a sublayer reads is h + conv(h): a short causal depthwise convolution beside the identity,
+                            its last taps - 1 inputs carried in the sequence's state slot
+  GatedOutputNorm           a sublayer's output times sigmoid(W h + b) of the sublayer's input, RMS-normed, added to the
+                            residual; the same launch norms the sum for the next sublayer
+  HeadDecayLinearAttention  linear attention with a matrix state per head that fades by one constant per head
+  ForgetGateLinearAttention linear attention whose per-channel forget gate f also writes: S <- diag(f) S + (1 - f) v^T
 
 Activations are fp32 tensors [rows, features]; matrices are stored in the serving dtype (bf16, or fp32 for the exact
 mode), vectors always in fp32.  A step's rows come with the metadata of utils/context.py: cu_seqlens_q, kv_lens (the
@@ -157,9 +163,15 @@ class ChannelDeltaMixer(nn.Module):
 
 
 class GroupedSparseMLP(nn.Module):
-    def __init__(self, width: int, ff: int, experts: int, identity: int, top_k: int, groups: int, keep: int):
+    """score: "softmax" over the router's outputs or each output's own "sigmoid"; group_value: a group of neighbouring
+    outputs is ranked by its best choice score ("max") or by the sum of its two best ("top2")."""
+
+    def __init__(self, width: int, ff: int, experts: int, identity: int, top_k: int, groups: int, keep: int,
+                 score: str = "softmax", group_value: str = "max"):
         super().__init__()
         self.E, self.n_out, self.top_k, self.groups, self.keep = experts, experts + identity, top_k, groups, keep
+        self.score_kind = {"softmax": _C.ROUTE_SOFTMAX, "sigmoid": _C.ROUTE_SIGMOID}[score]
+        self.group_kind = {"max": _C.ROUTE_GROUP_MAX, "top2": _C.ROUTE_GROUP_TOP2}[group_value]
         assert self.n_out % groups == 0 and 1 <= keep <= groups and top_k <= keep * (self.n_out // groups)
         self.router = _matrix(self.n_out, width)
         self.correction = _vector(self.n_out)
@@ -169,7 +181,8 @@ class GroupedSparseMLP(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         z = ops.gemm_any(x, self.router, exact=True)  # router logits in true 32-bit in every serving mode
-        ids, wts = ops.route_grouped(z, self.correction, self.top_k, self.groups, self.keep)
+        ids, wts = ops.route_grouped(z, self.correction, self.top_k, self.groups, self.keep, self.score_kind,
+                                     self.group_kind)
         offsets, pair_token, pair_index = ops.moe_sort(ids, self.n_out)
         P = ids.numel()
         act = ops.gemm_any_grouped(x, pair_token, self.gate, self.up, offsets, P, None, P)
@@ -248,14 +261,26 @@ class LatentAttention(nn.Module):
     per-head projections around it are batched GEMMs over head-major rows."""
 
     def __init__(self, width: int, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int, rot_dims: int,
-                 rot_base: float, scale: float, eps: float):
+                 rot_base: float, scale: float, eps: float, q_rank: int = 0, gate: bool = True, sink: bool = False):
+        """q_rank > 0: the queries come through a latent of their own, q = W_uq rms(W_dq h) * w_q (the down-projection
+        rides with the key/value one); gate: sigmoid output gate W_g h; sink: a learned logit per head in the softmax's
+        denominator.  rot_dim = 0: no rotated part - nothing in the layer depends on positions."""
         super().__init__()
         assert 0 <= rot_dims <= rot_dim and rot_dims % 2 == 0
-        self.H, self.D, self.R, self.Dv, self.C = heads, dim, rot_dim, vdim, kv_rank
+        self.H, self.D, self.R, self.Dv, self.C, self.Q = heads, dim, rot_dim, vdim, kv_rank, q_rank
         self.rot_dims, self.rot_base, self.scale, self.eps = rot_dims, rot_base, scale, eps
         # base^(-2 i / dims) in double, rounded once (a buffer, not a checkpoint tensor)
         self.register_buffer("inv_freq", rotary_inv_freq(rot_dims, rot_base), persistent=False)
-        self.qcg = MergedRows(width, {"q": heads * (dim + rot_dim), "dkv": kv_rank + rot_dim, "g": heads * vdim})
+        parts = {"dq": q_rank} if q_rank else {"q": heads * (dim + rot_dim)}
+        parts["dkv"] = kv_rank + rot_dim
+        if gate:
+            parts["g"] = heads * vdim
+        self.gated = gate
+        self.qcg = MergedRows(width, parts)
+        if q_rank:
+            self.q_norm = _vector(q_rank, 1.0)
+            self.uq = _matrix(heads * (dim + rot_dim), q_rank)
+        self.sink = _vector(heads) if sink else None
         self.c_norm = _vector(kv_rank, 1.0)
         self.uk_t = _matrix(heads, kv_rank, dim)   # W_uk,h transposed: the query-side projection into the latent space
         self.uv = _matrix(heads, vdim, kv_rank)
@@ -271,14 +296,18 @@ class LatentAttention(nn.Module):
         ctx, m = get_context(), self.qcg
         H, D, R, Dv, C = self.H, self.D, self.R, self.Dv, self.C
         y = m(h)
+        if self.Q:   # queries through their own latent: norm of the down-projection's columns, then the up-projection
+            q, q_off = ops.gemm_any(ops.add_rmsnorm_f32(m.cols(y, "dq"), None, 0.0, self.q_norm, self.eps), self.uq), 0
+        else:
+            q, q_off = y, m.offsets["q"][0]
         qx = torch.empty((h.shape[0], H * (C + R)), dtype=torch.float32, device=h.device)
-        ops.latent_prepare(y, m.offsets["q"][0], m.offsets["dkv"][0], H, D, R, C, self.rot_dims, self.inv_freq, self.c_norm,
+        ops.latent_prepare(y, q, q_off, m.offsets["dkv"][0], H, D, R, C, self.rot_dims, self.inv_freq, self.c_norm,
                            self.eps, ctx.cu_seqlens_q, ctx.kv_lens, self.cache, ctx.slot_mapping, qx)
-        ops.gemm_any_batched(m.cols(y, "q"), D + R, self.uk_t, qx, C + R)
+        ops.gemm_any_batched(q[:, q_off:q_off + H * (D + R)], D + R, self.uk_t, qx, C + R)
         o = ops.paged_attention_f32(qx, self.cache, self.cache, C + R, ctx.block_tables, ctx.cu_seqlens_q, ctx.kv_lens, H, 1,
-                                    C + R, C, ctx.block_size, CAUSAL, self.scale, _C.BIAS_NONE)
+                                    C + R, C, ctx.block_size, CAUSAL, self.scale, _C.BIAS_NONE, sink=self.sink)
         ov = torch.empty((h.shape[0], H * Dv), dtype=torch.float32, device=h.device)
-        ops.gemm_any_batched(o, C, self.uv, ov, Dv, gate=m.cols(y, "g"), gate_batch=Dv)
+        ops.gemm_any_batched(o, C, self.uv, ov, Dv, gate=m.cols(y, "g") if self.gated else None, gate_batch=Dv)
         return ops.gemm_any(ov, self.o)
 
 
@@ -351,3 +380,98 @@ class SharedSparseMLP(nn.Module):
             return ops.moe_combine_shared(y, ids, wts, h.shape[1])
         sh = ops.gemm_any(ops.gemm_any_act(h, self.shared_up, act=self.act), self.shared_down)
         return ops.moe_combine_shared(y, ids, wts, h.shape[1], sh, z[:, self.E:])
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# sandwich-normed families: gated residual branches, an input convolution, linear attention with a decayed state
+# ---------------------------------------------------------------------------------------------------------------------
+class InputConvolution(nn.Module):
+    """u = h + conv(h), conv(h)_t[c] = sum_j w[c, j] h_{t - (taps - 1) + j}[c] with zeros before the sequence's start.
+    The last taps - 1 rows of h live in the sequence's state slot `state` [slots, taps - 1, width]."""
+
+    def __init__(self, width: int, taps: int):
+        super().__init__()
+        assert 1 <= taps <= 17
+        self.taps = taps
+        self.weight = nn.Parameter(torch.zeros(width, taps, dtype=torch.float32), requires_grad=False)
+        self.state = torch.tensor([])
+
+    def state_shape(self, n_slots: int):
+        return (n_slots, max(self.taps - 1, 1), self.weight.shape[0])
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        ctx = get_context()
+        cu, kv, slots = ctx.cu_seqlens_q, ctx.kv_lens, ctx.state_slots
+        u = ops.causal_conv(h, self.weight, self.state, cu, kv, slots, silu=False, add_input=True)
+        ops.causal_conv_state(h, self.taps, self.state, cu, kv, slots)
+        return u
+
+
+class GatedOutputNorm(nn.Module):
+    """x <- x + rms(sigmoid(W_g h + b_g) * f(h)) * w, h being what the sublayer f was handed."""
+
+    def __init__(self, width: int, eps: float):
+        super().__init__()
+        self.eps = eps
+        self.gate, self.gate_b, self.weight = _matrix(width, width), _vector(width), _vector(width, 1.0)
+
+    def gate_of(self, h: torch.Tensor) -> torch.Tensor:
+        """-> W_g h + b_g (the sigmoid is taken where the gate is applied)"""
+        return ops.gemm_any_act(h, self.gate, bias=self.gate_b)
+
+    def add_to(self, residual: torch.Tensor, y: torch.Tensor, gate_pre: torch.Tensor, next_norm: torch.Tensor | None):
+        """residual += rms(y * sigmoid(gate_pre)) * w in place; -> rms(residual) * next_norm (None without one)"""
+        return ops.gated_norm_add_f32(residual, y, gate_pre, self.weight, self.eps, next_norm)
+
+
+class _LinearAttentionState(nn.Module):
+    def state_shape(self, n_slots: int):
+        return (n_slots, ops.linear_attention_state_elems(self.H, self.D, self.Dv))
+
+
+class HeadDecayLinearAttention(_LinearAttentionState):
+    """q = silu(W_q u), k = silu(W_k u), v = silu(W_v u); per head S <- decay_h S + k v^T, o = S^T q; the heads' read-outs
+    are RMS-normed TOGETHER (weight [heads * vdim]), times sigmoid(W_g u), then W_o.  fp32 state per sequence slot."""
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, decay, eps: float):
+        super().__init__()
+        assert len(decay) == heads
+        self.H, self.D, self.Dv, self.eps = heads, dim, vdim, eps
+        self.qkvg = MergedRows(width, {"q": heads * dim, "k": heads * dim, "v": heads * vdim, "g": heads * vdim})
+        self.register_buffer("decay", torch.tensor([float(d) for d in decay], dtype=torch.float64).to(torch.float32),
+                             persistent=False)
+        self.norm = _vector(heads * vdim, 1.0)
+        self.o = _matrix(width, heads * vdim)
+        self.state = torch.tensor([])
+
+    def forward(self, u: torch.Tensor) -> torch.Tensor:
+        ctx, m = get_context(), self.qkvg
+        y = m(u)
+        off = m.offsets
+        o = ops.linear_attention(y, off["q"][0], off["k"][0], off["v"][0], (_C.ACT_SILU,) * 3, _C.DECAY_HEAD, self.decay, None,
+                                 None, m.cols(y, "g"), self.norm, 1, self.state, ctx.cu_seqlens_q, ctx.kv_lens,
+                                 ctx.state_slots, self.H, self.D, self.Dv, self.eps)
+        return ops.gemm_any(o, self.o)
+
+
+class ForgetGateLinearAttention(_LinearAttentionState):
+    """q = silu(W_q u), v = W_v u, f = l + (1 - l) sigmoid(W_f u + b_f) with a lower bound l per channel; per head
+    S <- diag(f) S + (1 - f) v^T, o = S^T q; each head's read-out is RMS-normed over its value channels (one weight [vdim]
+    for all heads), then W_o.  fp32 state per sequence slot."""
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, eps: float):
+        super().__init__()
+        self.H, self.D, self.Dv, self.eps = heads, dim, vdim, eps
+        self.qfv = MergedRows(width, {"q": heads * dim, "f": heads * dim, "v": heads * vdim})
+        self.f_bias, self.lower, self.norm = _vector(heads * dim), _vector(heads * dim), _vector(vdim, 1.0)
+        self.o = _matrix(width, heads * vdim)
+        self.state = torch.tensor([])
+
+    def forward(self, u: torch.Tensor) -> torch.Tensor:
+        ctx, m = get_context(), self.qfv
+        y = m(u)
+        off = m.offsets
+        o = ops.linear_attention(y, off["q"][0], off["f"][0], off["v"][0], (_C.ACT_SILU, _C.ACT_NONE, _C.ACT_NONE),
+                                 _C.DECAY_FORGET, None, self.f_bias, self.lower, None, self.norm, self.H, self.state,
+                                 ctx.cu_seqlens_q, ctx.kv_lens, ctx.state_slots, self.H, self.D, self.Dv, self.eps)
+        return ops.gemm_any(o, self.o)

@@ -2,6 +2,7 @@
 The decoder families of the reference that share the paged-KV decode path: Qwen3 / Qwen2 (one class,
 qwen3.py:70-72 switches between q/k norm and qkv bias), Llama (models/llama.py) and Qwen3-MoE
 (models/qwen3_moe.py).  MiniCPM and Qwen3-VL are outside this package's scope."""
+from nanovllm.models.felolorn import FelolornConfig, FelolornForCausalLM
 from nanovllm.models.gazutar import GazutarConfig, GazutarForCausalLM
 from nanovllm.models.llama import LlamaForCausalLM
 from nanovllm.models.qwen3 import Qwen3ForCausalLM
@@ -15,12 +16,14 @@ model_dict = {
     "Qwen3MoeForCausalLM": Qwen3MoeForCausalLM,
     "Gazutar": GazutarForCausalLM,
     "Zedirax": ZediraxForCausalLM,
+    "Felolorn": FelolornForCausalLM,
 }
 
 # designs whose config.json is not a transformers configuration: {"architecture": <name>, ...} -> the reader of it
 native_configs = {
     "Gazutar": GazutarConfig,
     "Zedirax": ZediraxConfig,
+    "Felolorn": FelolornConfig,
 }
 
 

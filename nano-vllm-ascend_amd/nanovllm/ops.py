@@ -985,14 +985,14 @@ def gemm_any_grouped(x, x_rows, w, w2, group_offsets, rows_max: int, y_rows, y_r
     return y
 
 
-def embedding_f32(ids, table, out=None) -> torch.Tensor:
+def embedding_f32(ids, table, out=None, scale: float = 1.0) -> torch.Tensor:
     require_gpu(ids, table)
     assert ids.dtype == torch.int64 and ids.is_contiguous() and table.is_contiguous()
     if out is None:
         out = torch.empty((ids.numel(), table.shape[1]), dtype=_F32, device=table.device)
     assert out.shape == (ids.numel(), table.shape[1]) and out.dtype == _F32 and out.is_contiguous()
     check(lib.mi_embedding_f32(ptr(ids), ptr(table), _dt(table), ptr(out), ids.numel(), table.shape[1], table.shape[0],
-                               stream()), "mi_embedding_f32")
+                               float(scale), stream()), "mi_embedding_f32")
     return out
 
 
@@ -1045,6 +1045,21 @@ def causal_conv_silu(x, w, state, cu_q, kv_lens, slot_ids) -> torch.Tensor:
     return y
 
 
+def causal_conv(x, w, state, cu_q, kv_lens, slot_ids, silu: bool = False, add_input: bool = False) -> torch.Tensor:
+    """act(depthwise causal conv of x) (+ x); `state` [slots, taps - 1, C] is READ here and advanced by
+    causal_conv_state()."""
+    require_gpu(x, w, state)
+    _f32(x, w, state)
+    _i32(cu_q, kv_lens, slot_ids)
+    rows, C = x.shape
+    taps = w.shape[1]
+    assert w.shape[0] == C and w.is_contiguous() and state.is_contiguous() and state.shape[1:] == (max(taps - 1, 1), C)
+    y = torch.empty((rows, C), dtype=_F32, device=x.device)
+    check(lib.mi_causal_conv(ptr(x), x.stride(0), ptr(w), taps, ptr(state), ptr(cu_q), ptr(kv_lens), ptr(slot_ids),
+                             kv_lens.numel(), rows, C, int(silu), int(add_input), ptr(y), C, stream()), "mi_causal_conv")
+    return y
+
+
 def causal_conv_state(x, taps: int, state, cu_q, kv_lens, slot_ids) -> None:
     require_gpu(x, state)
     _f32(x, state)
@@ -1080,14 +1095,15 @@ def channel_delta(qkv, q_off: int, k_off: int, v_off: int, beta_pre, decay_pre, 
     return out
 
 
-def route_grouped(logits, correction, top_k: int, n_groups: int, keep: int):
+def route_grouped(logits, correction, top_k: int, n_groups: int, keep: int, score_kind: int = _C.ROUTE_SOFTMAX,
+                  group_kind: int = _C.ROUTE_GROUP_MAX):
     require_gpu(logits, correction)
     _f32(logits, correction)
     T, n = logits.shape
     ids = torch.empty((T, top_k), dtype=torch.int32, device=logits.device)
     wts = torch.empty((T, top_k), dtype=_F32, device=logits.device)
-    check(lib.mi_route_grouped(ptr(logits), logits.stride(0), ptr(correction), T, n, top_k, n_groups, keep, ptr(ids),
-                               ptr(wts), stream()), "mi_route_grouped")
+    check(lib.mi_route_grouped(ptr(logits), logits.stride(0), ptr(correction), T, n, top_k, n_groups, keep,
+                               int(score_kind), int(group_kind), ptr(ids), ptr(wts), stream()), "mi_route_grouped")
     return ids, wts
 
 
@@ -1170,10 +1186,12 @@ def gemm_any_batched(x, x_batch: int, w, out, out_batch: int, gate=None, gate_ba
 
 def paged_attention_f32(q, k_cache, v_cache, ldv: int, block_tables, cu_q, kv_lens, H: int, G: int, D: int, Dv: int,
                         block_size: int, window: int, scale: float, bias_kind: int = _C.BIAS_NONE, bias_p1=None, bias_p2=None,
-                        gate=None) -> torch.Tensor:
-    """Paged causal attention over fp32 queries; see mi_paged_attention_f32 (bias kinds, values inside the key rows)."""
+                        gate=None, sink=None) -> torch.Tensor:
+    """Paged causal attention over fp32 queries; see mi_paged_attention_f32 (bias kinds, values inside the key rows, a
+    sink logit per head in the softmax's denominator)."""
     require_gpu(q, k_cache, v_cache, block_tables, cu_q, kv_lens)
-    _f32(q, gate, bias_p1, bias_p2)
+    _f32(q, gate, bias_p1, bias_p2, sink)
+    assert sink is None or (sink.numel() == H and sink.is_contiguous())
     _i32(block_tables, cu_q, kv_lens)
     rows, n_seqs = q.shape[0], kv_lens.numel()
     assert q.shape[1] >= H * D and cu_q.numel() == n_seqs + 1 and block_tables.shape[0] >= n_seqs
@@ -1186,7 +1204,8 @@ def paged_attention_f32(q, k_cache, v_cache, ldv: int, block_tables, cu_q, kv_le
     check(lib.mi_paged_attention_f32(ptr(q), q.stride(0), ptr(k_cache), ptr(v_cache), int(ldv), _dt(k_cache),
                                      ptr(block_tables), block_tables.shape[1], ptr(cu_q), ptr(kv_lens), n_seqs, rows, H, G,
                                      D, Dv, block_size, int(min(window, 2 ** 31 - 1)), float(scale), int(bias_kind),
-                                     ptr(bias_p1), ptr(bias_p2), ptr(gate), gate.stride(0) if gate is not None else 0,
+                                     ptr(bias_p1), ptr(bias_p2), ptr(sink), ptr(gate),
+                                     gate.stride(0) if gate is not None else 0,
                                      ptr(out), out.stride(0), ptr(ws), ws.numel() if ws is not None else 0, stream()),
           "mi_paged_attention_f32")
     return out
@@ -1253,16 +1272,19 @@ def kv_store_temp(proj, q_off: int, k_off: int, v_off: int, temp_coef: float, te
                                G, D, Dv, block_size, stream()), "mi_kv_store_temp")
 
 
-def latent_prepare(proj, q_off: int, c_off: int, H: int, D: int, R: int, C: int, rot_dims: int, inv_freq, norm_w,
+def latent_prepare(proj, q, q_off: int, c_off: int, H: int, D: int, R: int, C: int, rot_dims: int, inv_freq, norm_w,
                    eps: float, cu_q, kv_lens, cache, slots, qx) -> None:
-    require_gpu(proj, cache, slots, qx)
-    _f32(proj, norm_w, qx, inv_freq)
+    """proj: the rows holding the key/value latent at c_off; q: the rows holding the query heads at q_off (may be proj)."""
+    require_gpu(proj, q, cache, slots, qx)
+    _f32(proj, q, norm_w, qx, inv_freq)
     _i32(slots, cu_q, kv_lens)
     rows = proj.shape[0]
     assert inv_freq.is_cuda and inv_freq.numel() >= rot_dims // 2
     assert slots.numel() == rows and norm_w.numel() == C and cache.shape[-1] == C + R and cache.is_contiguous()
-    assert qx.shape == (rows, H * (C + R)) and max(q_off + H * (D + R), c_off + C + R) <= proj.shape[1]
-    check(lib.mi_latent_prepare(ptr(proj), proj.stride(0), q_off, c_off, H, D, R, C, int(rot_dims), ptr(inv_freq),
+    assert qx.shape == (rows, H * (C + R)) and c_off + C + R <= proj.shape[1]
+    assert q.shape[0] == rows and q_off + H * (D + R) <= q.shape[1]
+    check(lib.mi_latent_prepare(ptr(proj), proj.stride(0), ptr(q), q.stride(0), q_off, c_off, H, D, R, C, int(rot_dims),
+                                ptr(inv_freq),
                                 ptr(norm_w), float(eps), ptr(cu_q), ptr(kv_lens), kv_lens.numel(), ptr(cache), _dt(cache),
                                 ptr(slots), ptr(qx), qx.stride(0), rows, stream()), "mi_latent_prepare")
 
@@ -1292,4 +1314,56 @@ def moe_combine_shared(y, ids, wts, width: int, shared=None, shared_gate=None) -
                                     shared.stride(0) if shared is not None else 0, ptr(shared_gate),
                                     shared_gate.stride(0) if shared_gate is not None else 0, ptr(out), width, stream()),
           "mi_moe_combine_shared")
+    return out
+
+
+
+# ---- sandwich-normed families with gated residual branches, decayed linear attention (csrc/seqmix.hip)
+def gated_norm_add_f32(res, y, gate_pre, w_post, eps: float, w_next=None):
+    """res += rms(y * sigmoid(gate_pre)) * w_post in place (gate_pre None: no gate); w_next given: returns
+    rms(res) * w_next, else None."""
+    require_gpu(res, y, w_post)
+    _f32(res, y, gate_pre, w_post, w_next)
+    rows, width = res.shape
+    assert y.shape == res.shape and w_post.numel() == width and (gate_pre is None or gate_pre.shape == res.shape)
+    out = None
+    if w_next is not None:
+        assert w_next.numel() == width
+        out = torch.empty((rows, width), dtype=_F32, device=res.device)
+    check(lib.mi_gated_norm_add_f32(ptr(res), res.stride(0), ptr(y), y.stride(0), ptr(gate_pre),
+                                    gate_pre.stride(0) if gate_pre is not None else 0, ptr(w_post), float(eps), ptr(w_next),
+                                    ptr(out), width, rows, width, stream()), "mi_gated_norm_add_f32")
+    return out
+
+
+def linear_attention_state_elems(H: int, D: int, Dv: int) -> int:
+    """Floats of state per sequence slot (the kernel keeps it in its own thread-order layout)."""
+    n = lib.mi_linear_attention_state_elems(H, D, Dv)
+    if n < 0:
+        raise _C.MiError(f"linear attention: {D} key channels per head are beyond the compiled kernels (<= 256)")
+    return n
+
+
+def linear_attention(proj, q_off: int, k_off: int, v_off: int, acts, decay_kind: int, decay, f_bias, lower, gate_pre, norm_w,
+                     norm_groups: int, state, cu_q, kv_lens, slot_ids, H: int, D: int, Dv: int, eps: float) -> torch.Tensor:
+    """S <- diag(a) S + k v^T, o = S^T q per head over the step's rows (see mi_linear_attention); acts = the (q, k, v)
+    activations; returns the normed (and gated) read-out [rows, H * Dv]."""
+    require_gpu(proj, state)
+    _f32(proj, decay, f_bias, lower, gate_pre, norm_w, state)
+    _i32(cu_q, kv_lens, slot_ids)
+    rows = proj.shape[0]
+    assert state.is_contiguous() and state.shape[1] == linear_attention_state_elems(H, D, Dv), state.shape
+    assert max(q_off + H * D, k_off + H * D, v_off + H * Dv) <= proj.shape[1]
+    if decay_kind == _C.DECAY_HEAD:
+        assert decay.numel() == H and decay.is_contiguous()
+    else:
+        assert f_bias.numel() == H * D and lower.numel() == H * D
+    assert norm_w is None or norm_w.numel() == (H * Dv if norm_groups == 1 else Dv)
+    assert gate_pre is None or (gate_pre.shape[0] == rows and gate_pre.shape[1] >= H * Dv)
+    out = torch.empty((rows, H * Dv), dtype=_F32, device=proj.device)
+    check(lib.mi_linear_attention(ptr(proj), proj.stride(0), q_off, k_off, v_off, int(acts[0]), int(acts[1]), int(acts[2]),
+                                  int(decay_kind), ptr(decay), ptr(f_bias), ptr(lower), ptr(gate_pre),
+                                  gate_pre.stride(0) if gate_pre is not None else 0, ptr(norm_w), int(norm_groups),
+                                  ptr(state), ptr(cu_q), ptr(kv_lens), ptr(slot_ids), kv_lens.numel(), rows, H, D, Dv,
+                                  float(eps), ptr(out), out.stride(0), stream()), "mi_linear_attention")
     return out
