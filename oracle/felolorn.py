@@ -137,7 +137,7 @@ def forward(config, weights, tokens, dtype=torch.float64, collect=None):
     """Logits [T, vocab] of one sequence; `collect` (a list) receives the residual stream after every layer."""
     w = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in weights.items()}
     eps = float(config["norm"]["eps"])
-    x = w["embed"][torch.as_tensor(tokens, dtype=torch.long)] * float(config["embedding"]["scale"])
+    x = w["embed"][torch.as_tensor(tokens, dtype=torch.long)] * float((config.get("embedding") or {}).get("scale", 1.0))
     for i, spec in enumerate(config["layers"]):
         p = sub(w, f"l{i}.")
         h = rms_norm(x, p["norm1"], eps)
@@ -153,8 +153,8 @@ def forward(config, weights, tokens, dtype=torch.float64, collect=None):
         if collect is not None:
             collect.append(x)
     z = rms_norm(x, w["final.norm"], eps) @ w["embed"].T
-    cap = float(config["logit_softcap"])
-    return cap * torch.tanh(z / cap)
+    cap = float(config.get("logit_softcap") or 0.0)
+    return cap * torch.tanh(z / cap) if cap > 0 else z
 
 
 def tensor_shapes(config):

@@ -1,0 +1,682 @@
+"""Felolorn on the GPU against the plain statement of its mechanisms in oracle/felolorn.py (float64, one sequence at a time,
+dense scores, Python loops over time).  Small configurations of the tests' own making, random bf16-representable weights;
+where random weights would hide a fault the weights or inputs are shaped so that it shows.
+
+Bars (felolorn_harness.assert_close): float32 serving mode 5e-5 on every row (row-wise rms difference / rms of the expected
+logits), bfloat16 mode 2e-2 on the median row and 6e-2 on all but a few rows; two runs of the engine that differ only in the
+cut (portions, batch, pages, slots) 2e-5 in float32."""
+import pytest
+import torch
+
+from felolorn_harness import (F32_BAR, MIXED, Replay, assert_close, config, hgrn2, latent, lightning, moe, rel_err, tokens_of,
+                              with_mlp, write_model_dir)
+from oracle import felolorn as F
+
+pytestmark = pytest.mark.gpu
+
+CUT_BAR = 2e-5
+
+
+def expected(cfg, weights, tokens):
+    return F.forward(cfg, weights, tokens, dtype=torch.float64)
+
+
+@pytest.fixture(scope="module")
+def mixed_model():
+    w = F.random_model(MIXED, seed=3)
+    return MIXED, w, write_model_dir(MIXED, w)
+
+
+@pytest.fixture(scope="module", params=["float32", "bfloat16"])
+def mixed_replay(request, mixed_model):
+    r = Replay(mixed_model[2], request.param)
+    yield request.param, r
+    r.close()
+
+
+# ------------------------------------------------------------------------------------------------ each mechanism alone
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,layers,kw", [
+    ("lightning", [with_mlp(lightning(), None)], {}),
+    ("lightning_one_head_one_tap", [with_mlp(lightning(heads=1, dim=12, vdim=70), None)], {"taps": 1}),
+    ("lightning_wide_heads", [with_mlp(lightning(heads=2, dim=130, vdim=33), None)], {"taps": 5}),
+    ("lightning_no_decay", [with_mlp(lightning(heads=2, dim=16, vdim=16, decay=[1.0, 0.0]), None)], {}),
+    ("hgrn2", [with_mlp(hgrn2(), None)], {}),
+    ("hgrn2_many_small_heads", [with_mlp(hgrn2(heads=7, dim=4, vdim=6), None)], {"taps": 2}),
+    ("hgrn2_wide_heads", [with_mlp(hgrn2(heads=1, dim=200, vdim=64), None)], {}),
+    ("latent", [with_mlp(latent(), None)], {}),
+    ("latent_odd_sizes", [with_mlp(latent(heads=5, dim=10, vdim=7, kv_rank=13, q_rank=9), None)], {}),   # element-wise loads
+    ("latent_matrix_core_sizes", [with_mlp(latent(heads=4, dim=32, vdim=48, kv_rank=64, q_rank=32, scale=0.1), None)], {}),
+    ("latent_wide", [with_mlp(latent(heads=2, dim=40, vdim=24, kv_rank=288, q_rank=100, scale=0.05), None)], {"width": 72}),
+    ("latent_one_head", [with_mlp(latent(heads=1, dim=24, vdim=16, kv_rank=24, q_rank=8), None)], {}),
+    ("latent_many_heads", [with_mlp(latent(heads=20, dim=8, vdim=8, kv_rank=32, q_rank=16), None)], {}),
+    ("sparse_ff", [with_mlp(lightning(), moe())], {}),
+    ("sparse_ff_one_group", [with_mlp(hgrn2(), moe(ff=24, experts=5, top=2, count=1, keep=1))], {}),
+    ("sparse_ff_groups_of_one", [with_mlp(latent(), moe(ff=16, experts=6, top=2, count=6, keep=3))], {}),
+    ("sparse_ff_all_groups_all_experts", [with_mlp(lightning(), moe(ff=16, experts=4, top=4, count=2, keep=2))], {}),
+    ("sparse_ff_top1_many_experts", [with_mlp(hgrn2(), moe(ff=8, experts=70, top=1, count=7, keep=2))], {}),
+    ("no_cap_no_scale", [with_mlp(lightning(), moe())], {"cap": 0.0, "scale": 1.0}),
+    ("five_layers", [with_mlp(hgrn2(), None), with_mlp(lightning(), None)] * 2 + [with_mlp(latent(), None)], {}),
+])
+def test_mechanism_alone(name, layers, kw, dtype):
+    cfg = config(layers, **kw)
+    w = F.random_model(cfg, seed=11)
+    toks = tokens_of(45, cfg["vocab"], 5)
+    r = Replay(write_model_dir(cfg, w), dtype)
+    try:
+        r.runner.model.trace_layers = []
+        got = r.feed("a", toks, [45])
+        want_layers = []
+        want = F.forward(cfg, w, toks, collect=want_layers)
+        for i, (a, b) in enumerate(zip(r.runner.model.trace_layers, want_layers)):
+            assert_close(a.cpu(), b, dtype, f"the residual stream after layer {i}")
+        r.runner.model.trace_layers = None
+        assert_close(got, want, dtype)
+        # the same tokens again, one by one, through the cache / the state
+        assert_close(r.feed("b", toks, [3]), want, dtype)
+    finally:
+        r.close()
+
+
+# ------------------------------------------------------------------------------------------------ operators
+@pytest.mark.parametrize("T,n,top,count,keep", [(64, 12, 3, 4, 2), (40, 130, 6, 13, 4), (33, 512, 8, 8, 3), (5, 7, 7, 1, 1),
+                                                 (9, 66, 1, 66, 5), (50, 24, 4, 3, 3), (30, 10, 2, 5, 1)])
+@pytest.mark.parametrize("shift", [0.0, -3.0])
+def test_router_choices_and_weights(T, n, top, count, keep, shift):
+    """Sigmoid scores, the correction in the choice only, a group's value = its two best choice scores (a group of one: that
+    one), only the best groups eligible, un-renormalised weights; `shift`: all choice scores negative (an excluded expert
+    must count as minus infinity, not as 0); more outputs than a wave has lanes."""
+    from nanovllm import _C, ops
+
+    g = torch.Generator().manual_seed(n + top)
+    z = (torch.randn(T, n, generator=g) * 2).double().float()
+    corr = torch.randn(n, generator=g) * 0.3 + shift
+    h = torch.eye(n, dtype=torch.float64)
+    # the plain statement takes h and the router matrix: feed it the logits through an identity
+    idx, wts = F.route(z.double(), {"router": h, "correction": corr.double()},
+                       {"experts": n, "top": top, "groups": {"count": count, "keep": keep}})
+    ids, got = ops.route_grouped(z.cuda(), corr.cuda(), top, count, keep, _C.ROUTE_SIGMOID, _C.ROUTE_GROUP_TOP2)
+    assert torch.equal(ids.cpu().long().sort(-1).values, idx.sort(-1).values)
+    order = ids.cpu().long().argsort(-1)
+    assert torch.allclose(got.cpu().double().gather(1, order), wts.gather(1, idx.argsort(-1)), atol=1e-6)
+
+
+def test_router_softmax_and_best_choice_groups_still_there():
+    """The earlier kinds (softmax scores, a group ranked by its best choice) are the defaults."""
+    from nanovllm import ops
+
+    g = torch.Generator().manual_seed(1)
+    z, corr = torch.randn(20, 12, generator=g), torch.randn(12, generator=g) * 0.1
+    s = torch.softmax(z.double(), -1)
+    choice = (s + corr.double()).view(20, 3, 4)
+    best = choice.max(-1).values.topk(2, -1).indices
+    ok = torch.zeros(20, 3, dtype=torch.bool).scatter_(1, best, True)
+    want = choice.masked_fill(~ok.unsqueeze(-1), float("-inf")).view(20, 12).topk(2, -1).indices
+    ids, wts = ops.route_grouped(z.cuda(), corr.cuda(), 2, 3, 2)
+    assert torch.equal(ids.cpu().long(), want)
+    assert torch.allclose(wts.cpu().double(), s.gather(1, want), atol=1e-6)
+
+
+@pytest.mark.parametrize("rows,width", [(1, 24), (7, 80), (40, 256), (3, 2100), (5, 4500)])
+def test_gated_output_norm(rows, width):
+    """res += rms(y * sigmoid(gate)) * w and the next sublayer's norm of the sum, in one launch; rows wider than what a
+    thread keeps in registers; without gate, without the second norm."""
+    from nanovllm import ops
+
+    g = torch.Generator().manual_seed(width)
+    res, y, gate = torch.randn(rows, width, generator=g), torch.randn(rows, width, generator=g) * 3, torch.randn(rows, width, generator=g)
+    w, w2 = 1 + torch.randn(width, generator=g) * 0.1, 1 + torch.randn(width, generator=g) * 0.1
+    for use_gate in (True, False):
+        for use_next in (True, False):
+            v = y.double() * (torch.sigmoid(gate.double()) if use_gate else 1.0)
+            want = res.double() + F.rms_norm(v, w.double(), 1e-5)
+            r = res.clone().cuda()
+            h = ops.gated_norm_add_f32(r, y.cuda(), gate.cuda() if use_gate else None, w.cuda(), 1e-5, w2.cuda() if use_next else None)
+            assert (r.cpu().double() - want).abs().max() <= 1e-5
+            if use_next:
+                assert (h.cpu().double() - F.rms_norm(want, w2.double(), 1e-5)).abs().max() <= 1e-5
+            else:
+                assert h is None
+
+
+@pytest.mark.parametrize("taps", [1, 2, 4, 7])
+def test_input_convolution_with_a_carried_tail(taps):
+    """u = h + conv(h) over sequences that start in this step (zeros before position 0, whatever the slot holds) and
+    sequences that continue (the tail of the previous step), one row and many; then the new tail."""
+    from nanovllm import ops
+
+    g = torch.Generator().manual_seed(taps)
+    C, lens, first = 70, [9, 1, 2, 30], [6, 3, 1, 11]       # rows of the first and of the second step per sequence
+    w = torch.randn(C, taps, generator=g)
+    full = [torch.randn(a + b, C, generator=g) for a, b in zip(first, lens)]
+    want = [(f.double() + F.input_conv(f.double(), w.double())) for f in full]
+    state = torch.randn(6, max(taps - 1, 1), C, generator=g).cuda()
+    slots = torch.tensor([4, 0, 5, 2], dtype=torch.int32).cuda()
+    at = [0] * 4
+    for counts in (first, lens):
+        x = torch.cat([f[a:a + n] for f, a, n in zip(full, at, counts)])
+        cu = torch.tensor([0] + list(torch.tensor(counts).cumsum(0)), dtype=torch.int32).cuda()
+        kv = torch.tensor([a + n for a, n in zip(at, counts)], dtype=torch.int32).cuda()
+        u = ops.causal_conv(x.cuda(), w.cuda(), state, cu, kv, slots, silu=False, add_input=True).cpu().double()
+        ops.causal_conv_state(x.cuda(), taps, state, cu, kv, slots)
+        ref = torch.cat([wn[a:a + n] for wn, a, n in zip(want, at, counts)])
+        assert (u - ref).abs().max() <= 1e-5
+        at = [a + n for a, n in zip(at, counts)]
+
+
+@pytest.mark.parametrize("kind", ["head", "forget"])
+@pytest.mark.parametrize("H,D,Dv", [(3, 8, 12), (2, 20, 32), (1, 64, 70), (2, 100, 16), (1, 128, 40), (1, 200, 33), (1, 256, 32)])
+def test_linear_attention_walk(kind, H, D, Dv):
+    """The decayed-state walk against a loop over time: sequences of one row, of less and more than a batch of rows,
+    starting fresh in a used slot or continuing from the state the previous step left; slots of other sequences untouched;
+    every key-channel block size of the kernel, value widths that are no multiple of a column block."""
+    from nanovllm import _C, ops
+
+    g = torch.Generator().manual_seed(D + Dv)
+    first, second = [5, 1, 40, 17], [1, 3, 35, 16]
+    n_seq, width = 4, 2 * H * D + H * Dv + 3
+    q_off, k_off, v_off = 1, 1 + H * D, 3 + 2 * H * D
+    full = [torch.randn(a + b, width, generator=g) for a, b in zip(first, second)]
+    decay = torch.rand(H, generator=g) * 0.5 + 0.5
+    fb, low = torch.randn(H * D, generator=g), torch.rand(H * D, generator=g) * 0.9
+    gate_w = torch.randn(sum(first) + sum(second), H * Dv, generator=g)
+    norm_w = 1 + torch.randn(H * Dv if kind == "head" else Dv, generator=g) * 0.1
+
+    def loop(p):
+        p = p.double()
+        S, outs = torch.zeros(H, D, Dv, dtype=torch.float64), []
+        for t in range(p.shape[0]):
+            q = F.silu(p[t, q_off:q_off + H * D]).view(H, D)
+            if kind == "head":
+                k = F.silu(p[t, k_off:k_off + H * D]).view(H, D)
+                v = F.silu(p[t, v_off:v_off + H * Dv]).view(H, Dv)
+                a = decay.double().view(H, 1).expand(H, D)
+            else:
+                a = (low.double() + (1 - low.double()) * torch.sigmoid(p[t, k_off:k_off + H * D] + fb.double())).view(H, D)
+                k, v = 1 - a, p[t, v_off:v_off + H * Dv].view(H, Dv)
+            S = a.unsqueeze(-1) * S + k.unsqueeze(-1) * v.unsqueeze(-2)
+            outs.append(torch.einsum("hdv,hd->hv", S, q))
+        return torch.stack(outs)      # [T, H, Dv]
+
+    raw = [loop(f) for f in full]
+    state = torch.randn(6, ops.linear_attention_state_elems(H, D, Dv), generator=g).cuda()
+    before = state.clone()
+    slots = torch.tensor([3, 0, 5, 1], dtype=torch.int32).cuda()
+    at, row0 = [0] * n_seq, 0
+    for counts in (first, second):
+        x = torch.cat([f[a:a + n] for f, a, n in zip(full, at, counts)]).cuda()
+        cu = torch.tensor([0] + list(torch.tensor(counts).cumsum(0)), dtype=torch.int32).cuda()
+        kv = torch.tensor([a + n for a, n in zip(at, counts)], dtype=torch.int32).cuda()
+        gp = gate_w[row0:row0 + sum(counts)]
+        if kind == "head":
+            got = ops.linear_attention(x, q_off, k_off, v_off, (_C.ACT_SILU,) * 3, _C.DECAY_HEAD, decay.cuda(), None, None,
+                                       gp.cuda(), norm_w.cuda(), 1, state, cu, kv, slots, H, D, Dv, 1e-5)
+        else:
+            got = ops.linear_attention(x, q_off, k_off, v_off, (_C.ACT_SILU, _C.ACT_NONE, _C.ACT_NONE), _C.DECAY_FORGET, None,
+                                       fb.cuda(), low.cuda(), None, norm_w.cuda(), H, state, cu, kv, slots, H, D, Dv, 1e-5)
+        ref = torch.cat([r[a:a + n] for r, a, n in zip(raw, at, counts)])
+        if kind == "head":
+            ref = F.rms_norm(ref.reshape(-1, H * Dv), norm_w.double(), 1e-5) * torch.sigmoid(gp.double())
+        else:
+            ref = F.rms_norm(ref, norm_w.double(), 1e-5).reshape(-1, H * Dv)
+        assert (got.cpu().double() - ref).abs().max() <= 2e-5 * max(1.0, float(ref.abs().max())), kind
+        at = [a + n for a, n in zip(at, counts)]
+        row0 += sum(counts)
+    assert torch.equal(state[[2, 4]], before[[2, 4]]), "a slot of no sequence was written"
+
+
+def _paged(k, v, bs, g):
+    """k [n, G, D], v [n, G, Dv] -> caches with scattered pages and the block table"""
+    n = k.shape[0]
+    nb = -(-n // bs)
+    table = torch.randperm(nb + 3, generator=g)[:nb].to(torch.int32)
+    kc = torch.zeros(nb + 3, k.shape[1], bs, k.shape[2], dtype=k.dtype)
+    vc = torch.zeros(nb + 3, v.shape[1], bs, v.shape[2], dtype=v.dtype)
+    for p in range(n):
+        kc[table[p // bs], :, p % bs] = k[p]
+        vc[table[p // bs], :, p % bs] = v[p]
+    return kc, vc, table
+
+
+@pytest.mark.parametrize("cache", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("H,D,Dv,alias", [(4, 64, 48, True), (6, 96, 96, True), (3, 24, 24, True), (5, 13, 7, False), (2, 256, 224, True),
+                                          (20, 32, 32, True)])
+def test_attention_with_a_sink(cache, H, D, Dv, alias):
+    """The sink logit in every form of the paged attention: prompt portions (matrix cores over a bf16 cache, the 16-byte-load
+    form, the element-wise form) and decode steps (heads as columns with the keys split over workgroups and merged; four
+    waves per row), one key/value row for all heads, the values being the leading channels of the key rows.  Sinks from
+    far below to far above the scores."""
+    from nanovllm import _C, ops
+
+    g = torch.Generator().manual_seed(H * D + Dv)
+    bs, start, T = 16, 37, 150
+    n = start + T
+    k = torch.randn(n, 1, D, generator=g).to(cache)
+    v = k[..., :Dv] if alias else torch.randn(n, 1, Dv, generator=g).to(cache)
+    q = torch.randn(n, H, D, generator=g)
+    sink = torch.linspace(-6.0, 8.0, H)
+    s = torch.einsum("ihd,jd->hij", q.double(), k[:, 0].double()) * 0.2
+    hidden = torch.arange(n).view(1, n) > torch.arange(n).view(n, 1)
+    s = s.masked_fill(hidden, float("-inf"))
+    p = torch.softmax(torch.cat([s, sink.double().view(H, 1, 1).expand(H, n, 1)], -1), -1)[..., :n]
+    want = torch.einsum("hij,jd->ihd", p, v[:, 0].double())
+    kc, vc, table = _paged(k, v, bs, g)
+    kc_d = kc.cuda()
+    vc_d = kc_d if alias else vc.cuda()
+    ldv = D if alias else Dv
+    bar = 1e-4 * float(want.abs().max())
+    # a prompt's portion: rows start .. n - 1
+    got = ops.paged_attention_f32(q[start:].reshape(T, H * D).contiguous().cuda(), kc_d, vc_d, ldv, table.view(1, -1).cuda(),
+                                  torch.tensor([0, T], dtype=torch.int32).cuda(), torch.tensor([n], dtype=torch.int32).cuda(),
+                                  H, 1, D, Dv, bs, 2 ** 31 - 1, 0.2, _C.BIAS_NONE, sink=sink.cuda()).cpu().double().view(T, H, Dv)
+    assert (got - want[start:]).abs().max() <= bar
+    # decode steps: three sequences (prefixes of the same keys), one row each
+    lens = [1, 60, n]
+    tables = table.view(1, -1).repeat(3, 1)
+    qd = torch.stack([q[m - 1] for m in lens]).reshape(3, H * D).contiguous()
+    got = ops.paged_attention_f32(qd.cuda(), kc_d, vc_d, ldv, tables.cuda(), torch.arange(4, dtype=torch.int32).cuda(),
+                                  torch.tensor(lens, dtype=torch.int32).cuda(), H, 1, D, Dv, bs, 2 ** 31 - 1, 0.2,
+                                  _C.BIAS_NONE, sink=sink.cuda()).cpu().double().view(3, H, Dv)
+    assert (got - torch.stack([want[m - 1] for m in lens])).abs().max() <= bar
+
+
+@pytest.mark.parametrize("M", [1, 6, 40, 600])
+@pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32])
+def test_capped_head_projection_and_scaled_embedding(M, wdtype):
+    from nanovllm import _C, ops
+
+    g = torch.Generator().manual_seed(M)
+    N, K = 75, 52
+    x = torch.randn(M, K, generator=g)
+    w = torch.randn(N, K, generator=g).to(wdtype)
+    xr = x.bfloat16().double() if (wdtype == torch.bfloat16 and M > 8) else x.double()
+    z = xr @ w.double().T
+    got = ops.gemm_any_act(x.cuda(), w.cuda(), act=_C.ACT_SOFTCAP, alpha=11.0).cpu().double()
+    assert (got - 11.0 * torch.tanh(z / 11.0)).abs().max() <= 3e-5
+    ids = torch.randint(0, N, (M,), generator=g)
+    rows = ops.embedding_f32(ids.cuda(), w.cuda(), scale=3.5).cpu().double()
+    assert (rows - w.double()[ids] * 3.5).abs().max() <= 1e-6
+
+
+# ------------------------------------------------------------------------------------------------ cuts of one sequence
+def test_whole_prompt(mixed_model, mixed_replay):
+    cfg, w, _ = mixed_model
+    dtype, r = mixed_replay
+    toks = tokens_of(70, cfg["vocab"], 1)
+    assert_close(r.feed("p", toks, [70]), expected(cfg, w, toks), dtype)
+
+
+def test_prefill_then_token_by_token(mixed_model, mixed_replay):
+    """Decoding through pages and state slots: 20 prompt tokens, then 60 single tokens (across page borders at 32, 48, 64)."""
+    cfg, w, _ = mixed_model
+    dtype, r = mixed_replay
+    toks = tokens_of(80, cfg["vocab"], 2)
+    assert_close(r.feed("d", toks, [20]), expected(cfg, w, toks), dtype)
+
+
+def test_first_tokens_one_by_one(mixed_model, mixed_replay):
+    """A sequence that starts with single tokens: zero matrix states, a convolution that sees zeros before position 0."""
+    cfg, w, _ = mixed_model
+    dtype, r = mixed_replay
+    toks = tokens_of(12, cfg["vocab"], 3)
+    assert_close(r.feed("f", toks, []), expected(cfg, w, toks), dtype)
+
+
+@pytest.mark.parametrize("cuts", [[2, 2, 2, 3, 5, 2, 16, 15, 17, 2], [31, 2, 33], [16, 16, 16, 16], [1, 2, 1, 2, 40],
+                                  [6, 1, 7, 7, 6, 2, 14]])
+def test_portions(mixed_model, mixed_replay, cuts):
+    """Portions down to two tokens (shorter than the convolution reaches back), ending on and off page borders (16) and
+    the recurrence's batches of rows (16).  (The tokens are ones without a router near-tie in the first layers: in the
+    bfloat16 mode a row computed alone and the same row inside a long portion round differently, a near-tie then falls
+    either way with the cut, and a changed expert in an early layer travels on through every later layer's state.)"""
+    cfg, w, _ = mixed_model
+    dtype, r = mixed_replay
+    toks = tokens_of(75, cfg["vocab"], 6)
+    got = r.feed("c", toks, cuts)
+    assert_close(got, expected(cfg, w, toks), dtype)
+    if dtype == "float32":
+        assert rel_err(got, r.feed("w", toks, [75])) <= CUT_BAR
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_hundreds_of_keys(dtype):
+    """330 tokens (the attention kernels take keys 32 or 64 at a time: several rounds of the running softmax; the
+    recurrences walk in batches of 16 rows) with latent sizes of every attention kernel: whole, in portions, decoded."""
+    cfg = config([with_mlp(latent(heads=4, dim=32, vdim=48, kv_rank=64, q_rank=32, scale=0.1), None),
+                  with_mlp(lightning(), None),
+                  with_mlp(latent(heads=2, dim=12, vdim=10, kv_rank=22, q_rank=14), moe(ff=16, experts=6, top=2, count=3, keep=2)),
+                  with_mlp(hgrn2(), None),
+                  with_mlp(latent(heads=3, dim=16, vdim=16, kv_rank=40, q_rank=24), None)],
+                 width=96, vocab=61, taps=4)
+    w = F.random_model(cfg, seed=21)
+    toks = tokens_of(330, 61, 8)
+    want = expected(cfg, w, toks)
+    r = Replay(write_model_dir(cfg, w), dtype, pages=48)
+    try:
+        assert_close(r.feed("a", toks, [330]), want, dtype)
+        assert_close(r.feed("b", toks, [100, 3, 64, 65, 2, 70]), want, dtype)     # then 26 single tokens
+        assert_close(r.feed("c", toks, [140] + [1] * 100 + [90]), want, dtype)
+    finally:
+        r.close()
+
+
+def test_long_decoding(mixed_model, mixed_replay):
+    cfg, w, _ = mixed_model
+    dtype, r = mixed_replay
+    toks = tokens_of(300, cfg["vocab"], 6)
+    assert_close(r.feed("l", toks, [3]), expected(cfg, w, toks), dtype)
+
+
+# ------------------------------------------------------------------------------------------------ batches, pages, slots
+def test_unequal_batch_equals_alone(mixed_model, mixed_replay):
+    """Four requests of unequal length in mixed steps (portions beside single tokens, a request left out of a step, one that
+    ends and whose pages and slot the next one takes) against each request alone."""
+    cfg, w, _ = mixed_model
+    dtype, r = mixed_replay
+    V = cfg["vocab"]
+    seqs = {"a": tokens_of(50, V, 10), "b": tokens_of(7, V, 11), "c": tokens_of(33, V, 12), "d": tokens_of(21, V, 13),
+            "e": tokens_of(40, V, 14)}
+    plan = [
+        ([("a", 17), ("b", 2)], []),
+        ([("a", 1), ("b", 3), ("c", 30)], []),
+        ([("a", 1), ("c", 1), ("d", 21)], ["d"]),          # b left out
+        ([("a", 16), ("b", 2), ("c", 1), ("e", 2)], ["b"]),  # e takes d's slot and pages
+        ([("e", 30), ("c", 1), ("a", 15)], ["a", "c"]),
+        ([("e", 8)], ["e"]),
+    ]
+    at = {k: 0 for k in seqs}
+    got = {k: [] for k in seqs}
+    slots_seen = {}
+    for entries, end in plan:
+        step = [(k, seqs[k][at[k]:at[k] + n]) for k, n in entries]
+        out = r.step(step, end=[])
+        for k, n in entries:
+            got[k].append(out[k])
+            at[k] += n
+            slots_seen[k] = r.live[k].state_slot
+        for k in end:
+            assert at[k] == len(seqs[k])
+            r.scheduler.finish(r.live.pop(k))
+    assert slots_seen["e"] == slots_seen["d"], "the freed slot was not used again"
+    for k, toks in seqs.items():
+        both = torch.cat(got[k])
+        assert_close(both, expected(cfg, w, toks), dtype)
+        if dtype == "float32":
+            assert rel_err(both, r.feed(k + "_alone", toks, [len(toks)])) <= CUT_BAR, k
+
+
+def test_pages_and_slots_reused_without_clearing(mixed_model):
+    """A pool of exactly one request's pages and ONE state slot: every request runs in what the previous one left behind."""
+    cfg, w, d = mixed_model
+    r = Replay(d, "float32", pages=5, slots=1)
+    try:
+        for seed, cuts in ((20, [80]), (21, [40, 2, 30]), (22, [])):
+            toks = tokens_of(80 if cuts != [] else 20, cfg["vocab"], seed)
+            assert rel_err(r.feed("x", toks, cuts), expected(cfg, w, toks)) <= F32_BAR
+            assert len(r.scheduler.block_manager.free_block_ids) == 5 and r.scheduler.state_slots.free == [0]
+    finally:
+        r.close()
+
+
+# ------------------------------------------------------------------------------------------------ faults that random weights hide
+def _token_features(vocab, width):
+    e = torch.zeros(vocab, width)
+    e[:, 0] = 0.1
+    e[1, 1] = 0.6                                 # token 1 carries a large feature 1
+    for t in range(2, vocab):
+        e[t, 2 + t % 4] = 0.1
+    return e
+
+
+def _spiky_latent_model(sink):
+    """A latent attention whose keys and queries are a function of the token alone: the latent's channel 0 is large for
+    token 1 only, every query looks for it, and its score stands out by far more than hundreds of other keys and the sink
+    weigh together; the input convolution is switched off, the gates are half open."""
+    cfg = config([with_mlp(latent(heads=2, dim=8, vdim=12, kv_rank=16, q_rank=8, scale=1.0), None)], width=32, vocab=8, taps=2)
+    w = F.random_model(cfg, seed=6)
+    w["embed"] = _token_features(8, 32)
+    dq, uq, dkv, uk = torch.zeros(8, 32), torch.zeros(16, 8), torch.zeros(16, 32), torch.zeros(16, 16)
+    dq[0, 0] = 1.0                                # the query latent: the feature every token has
+    uq[0, 0] = uq[8, 0] = 6.0                     # channel 0 of both heads
+    dkv[0, 1] = 1.0                               # latent channel 0 = feature 1
+    dkv[1, 0] = 1.0
+    dkv[2:6, 2:6] = torch.eye(4)
+    uk[0, 0] = uk[8, 0] = 1.0
+    w.update({"l0.mix.dq": dq, "l0.mix.uq": uq, "l0.mix.dkv": dkv, "l0.mix.uk": uk})
+    w["l0.mix.dq.norm"], w["l0.mix.dkv.norm"], w["l0.norm1"] = torch.ones(8), torch.ones(16), torch.ones(32)
+    w["l0.mix.sink"] = torch.tensor([sink, sink - 3.0])
+    w["l0.canon1"] = torch.zeros(32, 2)
+    w["l0.rg1"], w["l0.rg1.b"] = torch.zeros(32, 32), torch.zeros(32)
+    return cfg, {k: v.bfloat16().float() for k, v in w.items()}
+
+
+def test_a_far_key_among_hundreds():
+    """One dominant key at position p; every later row's output is that key's value, hundreds of positions on, across many
+    pages: a page of the block table that is skipped, a chunk of keys that is dropped, or a first key that is lost shows at
+    full size.  In a prompt, in portions, decoded; the key at position 0, at a page's last and first slot."""
+    cfg, w = _spiky_latent_model(sink=0.5)
+    r = Replay(write_model_dir(cfg, w), "float32", pages=30)
+    try:
+        for p in (0, 15, 16, 130):
+            n = 400
+            toks = [2 + (i % 6) for i in range(n)]
+            toks[p] = 1
+            plain = [2 + (i % 6) for i in range(n)]
+            want, without = expected(cfg, w, toks), expected(cfg, w, plain)
+            assert rel_err(without[n - 1:], want[n - 1:]) > 0.05, "the far key has no influence: the test's weights are wrong"
+            for cuts in ([n], [p + 1, 2, 200, 2], [300] + [1] * 60 + [40], [129, 129, 129]):
+                assert rel_err(r.feed("s", toks, cuts), want) <= F32_BAR, (p, cuts)
+    finally:
+        r.close()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_sink_takes_its_share(dtype):
+    """A sink far above the scores of a short prefix and level with one dominant key later: leaving it out, scaling it or
+    counting it once per chunk of keys changes the rows by tens of percent."""
+    cfg, w = _spiky_latent_model(sink=4.0)
+    n = 200
+    toks = [2 + (i % 6) for i in range(n)]
+    toks[70] = 1
+    want = expected(cfg, w, toks)
+    no_sink = dict(w)
+    no_sink["l0.mix.sink"] = torch.tensor([-30.0, -30.0])
+    assert rel_err(expected(cfg, no_sink, toks)[60:80], want[60:80]) > 0.05, "the sink has no influence: the test's weights are wrong"
+    r = Replay(write_model_dir(cfg, w), dtype, pages=30)
+    try:
+        for cuts in ([n], [69, 2, 2, 100], [100] + [1] * 70 + [30]):
+            got = r.feed("k", toks, cuts)
+            if dtype == "float32":
+                assert rel_err(got, want) <= F32_BAR, cuts
+            else:
+                assert_close(got, want, dtype)
+    finally:
+        r.close()
+
+
+@pytest.mark.parametrize("kind", ["lightning", "hgrn2"])
+def test_far_write_survives_in_the_state(kind):
+    """A matrix state that hardly fades: what position 2 wrote still shows 150 tokens later; a state lost or cleared at a
+    portion's start, or a slot mixed up in a batch, shows at full size."""
+    if kind == "lightning":
+        cfg = config([with_mlp(lightning(heads=2, dim=16, vdim=20, decay=[0.9995, 0.998]), None)], width=48, vocab=31)
+        w = F.random_model(cfg, seed=9)
+    else:
+        cfg = config([with_mlp(hgrn2(heads=2, dim=16, vdim=20), None)], width=48, vocab=31)
+        w = F.random_model(cfg, seed=9)
+        w["l0.mix.lower"] = torch.full((32,), 0.996)
+    w = {k: v.bfloat16().float() for k, v in w.items()}
+    toks = tokens_of(160, 31, 7)
+    other = list(toks)
+    other[2] = (toks[2] + 1) % 31
+    want, want_other = expected(cfg, w, toks), expected(cfg, w, other)
+    assert rel_err(want_other[150:], want[150:]) > 1e-3, "the early token has no influence: the test's weights are wrong"
+    r = Replay(write_model_dir(cfg, w), "float32", pages=24)
+    try:
+        assert rel_err(r.feed("a", toks, [160]), want) <= F32_BAR
+        assert rel_err(r.feed("b", toks, [5, 70, 2, 2, 60]), want) <= F32_BAR
+        for cut in (40, 1):   # two sequences that differ in the early token only, side by side in every step
+            at, got = 0, {"x": [], "y": []}
+            while at < 160:
+                n = min(cut, 160 - at)
+                out = r.step([("y", other[at:at + n]), ("x", toks[at:at + n])])
+                got["x"].append(out["x"])
+                got["y"].append(out["y"])
+                at += n
+            for k in ("x", "y"):
+                r.scheduler.finish(r.live.pop(k))
+            assert rel_err(torch.cat(got["x"]), want) <= F32_BAR and rel_err(torch.cat(got["y"]), want_other) <= F32_BAR
+    finally:
+        r.close()
+
+
+def test_the_convolution_reaches_back_over_portion_edges():
+    """Five taps of which the OLDEST weighs most: a row's mixer input is mostly what the layer's norm gave four positions
+    earlier.  Portions of one to three tokens take all of it from the carried tail; a tail that is shifted by one, not
+    advanced by a short portion, or taken from another slot shows at full size."""
+    cfg = config([with_mlp(lightning(heads=2, dim=12, vdim=12), None), with_mlp(hgrn2(heads=2, dim=8, vdim=8), None)],
+                 width=40, vocab=29, taps=5)
+    w = F.random_model(cfg, seed=12)
+    for i in (0, 1):
+        c = torch.zeros(40, 5)
+        c[:, 0] = 4.0
+        w[f"l{i}.canon1"] = c
+    toks = tokens_of(40, 29, 3)
+    want = expected(cfg, w, toks)
+    flat = dict(w)
+    for i in (0, 1):
+        flat[f"l{i}.canon1"] = torch.zeros(40, 5)
+    assert rel_err(expected(cfg, flat, toks)[8:], want[8:]) > 0.05, "the convolution has no influence: the test's weights are wrong"
+    r = Replay(write_model_dir(cfg, w), "float32")
+    try:
+        for cuts in ([40], [4, 1, 1, 1, 2, 3, 2, 4, 5, 6], [1, 1, 1, 1, 1, 35], [3, 3, 3, 3, 3, 2, 2, 2, 19], []):
+            assert rel_err(r.feed("t", toks, cuts), want) <= F32_BAR, cuts
+        a, b = tokens_of(30, 29, 4), tokens_of(30, 29, 5)     # two sequences side by side, portions of two
+        got = {"a": [], "b": []}
+        for at in range(0, 30, 2):
+            out = r.step([("a", a[at:at + 2]), ("b", b[at:at + 2])])
+            got["a"].append(out["a"])
+            got["b"].append(out["b"])
+        for k in ("a", "b"):
+            r.scheduler.finish(r.live.pop(k))
+        assert rel_err(torch.cat(got["a"]), expected(cfg, w, a)) <= F32_BAR
+        assert rel_err(torch.cat(got["b"]), expected(cfg, w, b)) <= F32_BAR
+    finally:
+        r.close()
+
+
+def test_the_gate_reads_what_the_convolution_has_not_touched():
+    """The residual gate is a function of the sublayer's input BEFORE the input convolution: with a strong convolution
+    and steep gates, gating by the convolved input would move every row."""
+    cfg = config([with_mlp(hgrn2(heads=2, dim=8, vdim=8), moe(ff=16, experts=4, top=2, count=2, keep=1))], width=40, vocab=29, taps=3)
+    w = F.random_model(cfg, seed=13)
+    w["l0.canon1"] = torch.full((40, 3), 1.5)
+    w["l0.rg1"] = (w["l0.rg1"] * 6).bfloat16().float()
+    toks = tokens_of(30, 29, 6)
+    r = Replay(write_model_dir(cfg, w), "float32")
+    try:
+        assert rel_err(r.feed("g", toks, [11, 2]), expected(cfg, w, toks)) <= F32_BAR
+    finally:
+        r.close()
+
+
+# ------------------------------------------------------------------------------------------------ the engine's own entry point
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_llm(mixed_model, dtype):
+    """LLM.generate: the scheduler's prefill and decode steps, its page and slot managers, captured decode steps, the sampler.
+    Every generated token must be the plain model's best token given the same history (or within the sampler's bf16 logits
+    of it); in the bfloat16 mode a router's near-tie now and then moves a row by more than that: two of the sixty may differ."""
+    from nanovllm import LLM, SamplingParams
+
+    cfg, w, d = mixed_model
+    llm = LLM(d, dtype=dtype, kvcache_block_size=16, num_kvcache_blocks=40, max_num_seqs=3, max_model_len=256,
+              max_num_batched_tokens=256, warmup=False)
+    try:
+        assert llm.model_runner.row_graphs
+        prompts = [tokens_of(n, cfg["vocab"], 30 + n) for n in (5, 40, 17, 33, 2)]   # five requests over three slots
+        outs = llm.generate(prompts, SamplingParams(max_tokens=12, greedy=True, ignore_eos=True), use_tqdm=False)
+        assert len(outs) == 5
+        off = []
+        for prompt, out in zip(prompts, outs):
+            gen = out["token_ids"]
+            assert len(gen) == 12
+            logits = expected(cfg, w, prompt + gen)
+            for i, tok in enumerate(gen):
+                row = logits[len(prompt) - 1 + i]
+                if row.max() - row[tok] > 0.06:
+                    off.append((len(prompt), i, tok, int(row.argmax()), float(row.max() - row[tok])))
+        assert len(off) <= (0 if dtype == "float32" else 2), off
+    finally:
+        llm.exit()
+
+
+def test_captured_decode_steps_equal_eager(mixed_model):
+    """Decode steps replay hipGraphs padded to a batch bucket (3 live requests in the bucket of 4, the padded row writing the
+    spare state slot): same tokens and the same logits as eager launches, over several replays with eager prefill steps
+    between them."""
+    from nanovllm import LLM, SamplingParams
+
+    cfg, w, d = mixed_model
+    prompts = [tokens_of(n, cfg["vocab"], 70 + n) for n in (9, 31, 16, 5, 22)]
+    sp = SamplingParams(max_tokens=10, greedy=True, ignore_eos=True)
+    runs, logits = [], []
+    for eager in (True, False):
+        llm = LLM(d, dtype="float32", kvcache_block_size=16, num_kvcache_blocks=40, max_num_seqs=4, max_model_len=128,
+                  max_num_batched_tokens=128, warmup=False, enforce_eager=eager)
+        try:
+            assert bool(llm.model_runner.row_graphs) == (not eager)
+            runs.append([o["token_ids"] for o in llm.generate(prompts[:3], sp, use_tqdm=False)])
+            runs[-1] += [o["token_ids"] for o in llm.generate(prompts[3:], sp, use_tqdm=False)]
+            logits.append(llm.model_runner.last_logits.float().cpu().clone())
+        finally:
+            llm.exit()
+    assert runs[0] == runs[1]
+    assert rel_err(logits[1], logits[0]) <= CUT_BAR
+
+
+def test_engine_chunked_prefill_equals_whole_prompts(mixed_model):
+    """Config.chunked_prefill: the engine's own scheduler cuts prompts into portions (24 rows per step) and batches them
+    with the other requests' decoded tokens; the generated tokens are those of whole-prompt prefill steps."""
+    from nanovllm import LLM, SamplingParams
+
+    cfg, w, d = mixed_model
+    prompts = [tokens_of(n, cfg["vocab"], 90 + n) for n in (70, 9, 41, 3, 26)]
+    sp = SamplingParams(max_tokens=9, greedy=True, ignore_eos=True)
+    runs = []
+    for kw in (dict(max_num_batched_tokens=128), dict(max_num_batched_tokens=24, chunked_prefill=True)):
+        llm = LLM(d, dtype="float32", kvcache_block_size=16, num_kvcache_blocks=40, max_num_seqs=3, max_model_len=128,
+                  warmup=False, **kw)
+        try:
+            runs.append([o["token_ids"] for o in llm.generate(prompts, sp, use_tqdm=False)])
+        finally:
+            llm.exit()
+    assert runs[0] == runs[1]
+
+
+def test_trace_replay_program(mixed_model, tmp_path):
+    """bin/trace_run end to end: steps on standard input, logits files and `done` lines out; two requests in one step."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    cfg, w, d = mixed_model
+    toks, other = tokens_of(30, cfg["vocab"], 60), tokens_of(9, cfg["vocab"], 61)
+    steps = [{"step": 0, "entries": [{"id": "q", "tokens": toks[:20], "want": [0, 19]}], "end": []},
+             {"step": 1, "entries": [{"id": "q", "tokens": toks[20:29], "want": []}, {"id": "o", "tokens": other[:8], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "o", "tokens": other[8:], "want": [0]}, {"id": "q", "tokens": toks[29:], "want": [0]}],
+              "end": ["q", "o"]}]
+    repo = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, os.path.join(repo, "bin", "trace_run"), "--model", d, "--dtype", "float32",
+                        "--out", str(tmp_path), "--max-tokens", "128"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    want, want_o = expected(cfg, w, toks), expected(cfg, w, other)
+    got0 = torch.from_numpy(np.fromfile(tmp_path / "0.f32", dtype="<f4").reshape(2, -1))
+    got2 = torch.from_numpy(np.fromfile(tmp_path / "2.f32", dtype="<f4").reshape(2, -1))
+    assert not (tmp_path / "1.f32").exists()
+    assert rel_err(got0, want[[0, 19]]) <= F32_BAR
+    assert rel_err(got2[:1], want_o[[8]]) <= F32_BAR and rel_err(got2[1:], want[[29]]) <= F32_BAR
