@@ -1,5 +1,5 @@
 """Prefill and decode throughput of a model design beside the framework's closest existing model at equal size
-(`python bench.py --design gazutar | zedirax`): random weights, layer sizes that resemble a real model's, both models through the same
+(`python bench.py --design gazutar | zedirax | felolorn`): random weights, layer sizes that resemble a real model's, both models through the same
 engine entry points (add_request / step), each served the way the framework serves it (Qwen3-MoE: captured prefill and
 decode steps; Gazutar: what ModelRunner reports in `served_as`).
 
@@ -69,6 +69,44 @@ def zedirax_decode_weight_bytes(cfg: dict, batch: int) -> float:
         else:
             hit = min(ml["router"]["experts"], batch * ml["router"]["top"])
             n += hit * 2 * W * ml["expert"]["ff"] + (ml["router"]["experts"] + 1) * W + 2 * W * ml["shared"]["ff"]
+    return 2.0 * (n + cfg["vocab"] * W)
+
+
+def felolorn_config(s: dict) -> dict:
+    """Forget-gate linear attention / latent attention / head-decay linear attention / latent attention, every layer with
+    a group-routed sparse feed-forward (four groups, two kept).  The latent attention caches 256 channels per token for
+    all heads (what the Zedirax bench model caches), queries through a latent of half the model width."""
+    W, D, H = s["width"], s["dim"], s["heads"]
+    lat = {"type": "latent_attention", "mixer": {"heads": H, "dim": D, "vdim": D, "kv_rank": 256, "q_rank": W // 2, "scale": D ** -0.5}}
+    lin = {"type": "lightning", "mixer": {"heads": H, "dim": D, "vdim": D, "decay": [1.0 - 2.0 ** (-5 - 3 * h / H) for h in range(H)]}}
+    fgt = {"type": "hgrn2", "mixer": {"heads": H, "dim": D, "vdim": D}}
+    moe = {"kind": "moe", "expert": {"ff": s["ff"]},
+           "router": {"experts": s["experts"], "top": s["top"], "groups": {"count": 4, "keep": 2}}}
+    order = [fgt, lat, lin, lat]
+    return {"architecture": "Felolorn", "vocab": s["vocab"], "width": W, "norm": {"eps": 1e-6}, "canon": {"taps": 4},
+            "embedding": {"scale": W ** 0.5}, "logit_softcap": 30.0,
+            "layers": [dict(order[i % 4], mlp=moe) for i in range(s["layers"])]}
+
+
+def felolorn_decode_weight_bytes(cfg: dict, batch: int) -> float:
+    """bf16 weight bytes one decode step of `batch` rows streams (every projection incl. the two residual gates, the experts
+    the rows can reach, the tied table as the head)."""
+    W, n = cfg["width"], 0
+    for l in cfg["layers"]:
+        m = l["mixer"]
+        H, D, Dv = m["heads"], m["dim"], m["vdim"]
+        n += W * W                                                   # the mixer's residual gate
+        if l["type"] == "latent_attention":
+            C, Q = m["kv_rank"], m["q_rank"]
+            n += W * (Q + C) + Q * H * D + H * C * (D + Dv) + H * Dv * W
+        elif l["type"] == "lightning":
+            n += W * (2 * H * D + 2 * H * Dv) + H * Dv * W
+        else:
+            n += W * (2 * H * D + H * Dv) + H * Dv * W
+        ml = l["mlp"]
+        if ml is not None:
+            hit = min(ml["router"]["experts"], batch * ml["router"]["top"])
+            n += W * W + hit * 3 * W * ml["expert"]["ff"] + ml["router"]["experts"] * W
     return 2.0 * (n + cfg["vocab"] * W)
 
 
@@ -147,6 +185,8 @@ def main(args) -> dict:
     design = getattr(args, "design", None) or "gazutar"
     if design == "zedirax":
         return main_zedirax(args, batch, prompt_len)
+    if design == "felolorn":
+        return main_felolorn(args, batch, prompt_len)
     out = {"metric": "design_throughput", "design": "gazutar", "closest_model": "Qwen3MoeForCausalLM", "unit": "tokens/s",
            "dtype": "bf16", "data": "synthetic (random weights, random prompts)", "n_gpus": 1, "steps": args.steps,
            "warmup": args.warmup, "batch": batch, "prompt_len": prompt_len, "sizes": {}}
@@ -196,6 +236,39 @@ def main_zedirax(args, batch: int, prompt_len: int) -> dict:
             entry[label] = r
         if "zedirax" in entry and "gazutar" in entry:
             entry["zedirax_vs_gazutar"] = {k: entry["zedirax"][k] / entry["gazutar"][k] for k in ("prefill_tok_s", "decode_tok_s")}
+        out["sizes"][name] = entry
+    print(json.dumps(out), flush=True)
+    return out
+
+
+def main_felolorn(args, batch: int, prompt_len: int) -> dict:
+    """Felolorn beside Zedirax - the closest existing model: the same row-step engine path, fp32 residual with RMS norms,
+    a latent attention with one cached row per token, a recurrence in state slots, sparse feed-forwards - at equal width,
+    depth, heads, experts and vocabulary; Gazutar (the matrix-state recurrence and the group-limited router of the
+    framework) and Qwen3-MoE at that size ride along (`--design-models` picks)."""
+    out = {"metric": "design_throughput", "design": "felolorn", "closest_model": "Zedirax", "unit": "tokens/s",
+           "dtype": "bf16", "data": "synthetic (random weights, random prompts)", "n_gpus": 1, "steps": args.steps,
+           "warmup": args.warmup, "batch": batch, "prompt_len": prompt_len, "sizes": {}}
+    only_sizes = [x for x in getattr(args, "design_sizes", "").split(",") if x]
+    only_models = [x for x in getattr(args, "design_models", "").split(",") if x] or ["felolorn", "zedirax", "gazutar"]
+    for name, s in SIZES.items():
+        if only_sizes and name not in only_sizes:
+            continue
+        entry = {"shape": s}
+        fc, zc = felolorn_config(s), zedirax_config(s)
+        for label, cfg, wb in (("felolorn", fc, felolorn_decode_weight_bytes(fc, batch)),
+                               ("zedirax", zc, zedirax_decode_weight_bytes(zc, batch)),
+                               ("gazutar", gazutar_config(s), decode_weight_bytes(s, batch, True)),
+                               ("qwen3_moe", qwen3_moe_config(s), decode_weight_bytes(s, batch, False))):
+            if label not in only_models:
+                continue
+            r = run_model(cfg, batch, prompt_len, args.steps, args.warmup)
+            r["decode_weight_bytes"] = wb
+            r["decode_weight_roofline_frac"] = wb / (r["ms_per_decode_step"] * 1e-3) / HBM_BYTES_PER_S
+            entry[label] = r
+        for other in ("zedirax", "gazutar"):
+            if "felolorn" in entry and other in entry:
+                entry["felolorn_vs_" + other] = {k: entry["felolorn"][k] / entry[other][k] for k in ("prefill_tok_s", "decode_tok_s")}
         out["sizes"][name] = entry
     print(json.dumps(out), flush=True)
     return out

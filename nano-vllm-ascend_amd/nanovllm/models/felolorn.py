@@ -68,7 +68,8 @@ class FelolornLayer(nn.Module):
             self.mix = LatentAttention(W, H, D, 0, Dv, int(m["kv_rank"]), 0, 1.0, float(m["scale"]), eps,
                                        q_rank=int(m["q_rank"]), gate=False, sink=True)
         elif self.kind == "lightning":
-            self.mix = HeadDecayLinearAttention(W, H, D, Dv, m["decay"], eps)
+            decay = m["decay"]
+            self.mix = HeadDecayLinearAttention(W, H, D, Dv, decay if isinstance(decay, (list, tuple)) else [decay] * H, eps)
         elif self.kind == "hgrn2":
             self.mix = ForgetGateLinearAttention(W, H, D, Dv, eps)
         else:

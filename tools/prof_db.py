@@ -4,6 +4,22 @@ import sqlite3
 import sys
 
 
+def demangle(names):
+    """Readable kernel names where the trace holds mangled ones (c++filt of the toolchain, if there is one)."""
+    import shutil
+    import subprocess
+
+    exe = shutil.which("c++filt") or shutil.which("llvm-cxxfilt")
+    if not exe:
+        return list(names)
+    stripped = [n[:-3] if n.endswith(".kd") else n for n in names]
+    try:
+        out = subprocess.run([exe], input="\n".join(stripped), capture_output=True, text=True, timeout=60).stdout.split("\n")
+    except (OSError, subprocess.SubprocessError):
+        return list(names)
+    return out[:len(stripped)] if len(out) >= len(stripped) else list(names)
+
+
 def main(path, top=30):
     db = sqlite3.connect(path)
     cur = db.cursor()
@@ -16,7 +32,8 @@ def main(path, top=30):
     rows = list(cur.execute(q))
     total = sum(r[5] for r in cur.execute(f"select 0,0,0,0,0,sum(end-start)/1000.0 from {kd}"))
     print(f"{'kernel':100s} {'calls':>7s} {'avg_us':>9s} {'min_us':>9s} {'max_us':>9s} {'total_us':>11s} {'%':>6s}")
-    for r in rows:
+    for name, r in zip(demangle([r[0] for r in rows]), rows):
+        r = (name,) + tuple(r[1:])
         print(f"{r[0][:100]:100s} {r[1]:7d} {r[2]:9.2f} {r[3]:9.2f} {r[4]:9.2f} {r[5]:11.1f} {100 * r[5] / total:6.2f}")
 
 
