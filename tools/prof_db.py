@@ -77,7 +77,8 @@ def window(path, anchor_substr, n_anchor, label):
         prev_end = max(prev_end, en)
     print(f"{label}: {n_anchor} x *{anchor_substr}* first start -> last end: {span:.1f} us "
           f"({span / max(1, n_anchor - 1) :.1f} us per anchor interval), kernels busy {busy:.1f} us, idle gaps {gaps:.1f} us")
-    for name, (cnt, tot) in sorted(per.items(), key=lambda kv: -kv[1][1])[:14]:
+    top = sorted(per.items(), key=lambda kv: -kv[1][1])[:26]
+    for name, (_, (cnt, tot)) in zip(demangle([k for k, _ in top]), top):
         print(f"   {name[:96]:96s} {cnt:5d} {tot / cnt:9.2f} us avg {tot:10.1f} us {100 * tot / span:5.1f} %")
 
 
