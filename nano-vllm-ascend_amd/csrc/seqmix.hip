@@ -1610,52 +1610,64 @@ __global__ __launch_bounds__(256) void gated_norm_add_f32_kernel(float* __restri
 //   MI_DECAY_HEAD    a_t = decay[h] for every key channel of head h and every row; q, k, v = act(projection)
 //   MI_DECAY_FORGET  a_t = f_t = lower + (1 - lower) * sigmoid(z_t + f_bias) per key channel (z at k_off), and what is
 //                    written is k_t = 1 - f_t: the forget gate also decides how much of v_t enters
-// The walk is channel_delta_kernel's: a workgroup = 32 value columns of one (sequence, head); a column is held by a quad
-// of lanes, lane r of it keeping the key channels (4 jj + r) * 4 + e in registers for the whole walk over the step's
-// rows; the rows' vectors of 16 rows at a time go through LDS, loaded one batch ahead as raw projections and turned into
-// q / k / a (activations, gate) on their way into LDS - no separate preparation launch; sums over the key channels end
-// in two DPP steps inside the quad.  The state lives in memory in thread order ([slot][head][column block][DR][128]).
-template <int DR, int DECAY>
-__global__ __launch_bounds__(kDeltaThreads) void linear_attention_kernel(
+// The walk has channel_delta_kernel's shape with SIXTEEN lanes per value column (the rule has one pass over the state per
+// row where the delta rule has two, and a prompt step's few (sequence, head) units should put two waves on every SIMD:
+// measured on 8 sequences x 1024 rows x 8 heads x 128 x 128 channels, 4 / 8 / 16 lanes per column: 785 / 417 / 304 us):
+// a workgroup = 32 value columns of one (sequence, head) = 512 threads; lane r of a column's sixteen keeps the key
+// channels (16 jj + r) * 4 + e in registers for the whole walk over the step's rows; the rows' vectors of 16 rows at a
+// time go through LDS, loaded one batch ahead as raw projections (32 lanes per row) and turned into q / k / a
+// (activations, gate, lower bound) on their way into LDS - no separate preparation launch; the sum over the key channels
+// ends in four DPP steps inside a 16-lane row.  The state lives in memory as [slot][head][column block][key channel / 4]
+// [32 columns][4]: a thread's four channels of a column are one 16-byte piece, a wave's loads whole 256-byte runs.
+constexpr int kLinLanes = 16, kLinThreads = kLinLanes * kDeltaCols, kLinStage = kLinThreads / kDeltaRows;
+static_assert(kLinStage * kDeltaRows == kLinThreads && kDeltaCols % kLinStage == 0, "whole staging lanes per row");
+static_assert(kLinLanes == 16, "the read-out's butterfly (1, 2, 4, 8) spans a column's lanes");
+
+template <int DR, int DECAY>  // DR: key channels per lane (the head's channels padded to kLinLanes * DR)
+__global__ __launch_bounds__(kLinThreads) void linear_attention_kernel(
     const float* __restrict__ proj, int64_t ld, int q_off, int k_off, int v_off, int q_act, int k_act, int v_act,
     const float* __restrict__ decay, const float* __restrict__ f_bias, const float* __restrict__ lower,
     float* __restrict__ state, const int32_t* __restrict__ cu_q, const int32_t* __restrict__ kv_lens,
     const int32_t* __restrict__ slot_ids, int H, int D, int Dv, float* __restrict__ out, int64_t ldo) {
-  constexpr int DP = 4 * DR;  // padded key channels
+  constexpr int DP = kLinLanes * DR;  // padded key channels
   constexpr bool FORGET = DECAY == MI_DECAY_FORGET;
   __shared__ __attribute__((aligned(16))) float qs[kDeltaRows][DP];
   __shared__ __attribute__((aligned(16))) float ks[kDeltaRows][DP];
   __shared__ __attribute__((aligned(16))) float gs[FORGET ? kDeltaRows : 1][DP];
   __shared__ float vs[kDeltaRows][kDeltaCols];
   const int s = blockIdx.x, h = blockIdx.y, cb = blockIdx.z;
-  const int tid = threadIdx.x, r = tid & 3, col = tid >> 2;
+  const int tid = threadIdx.x, r = tid & (kLinLanes - 1), col = tid / kLinLanes;
   const int c = cb * kDeltaCols + col;
   const int r0 = cu_q[s], n = cu_q[s + 1] - r0;
   if (n == 0) return;
   const int start = kv_lens[s] - n;
-  float* slot = state + (((int64_t)slot_ids[s] * H + h) * gridDim.z + cb) * DR * kDeltaThreads;
+  float* slot = state + (((int64_t)slot_ids[s] * H + h) * gridDim.z + cb) * DP * kDeltaCols;
   float st[DR];
 #pragma unroll
-  for (int ii = 0; ii < DR; ++ii) st[ii] = start > 0 ? slot[ii * kDeltaThreads + tid] : 0.f;
+  for (int jj = 0; jj < DR / 4; ++jj) {
+    float4 v4{0.f, 0.f, 0.f, 0.f};
+    if (start > 0) v4 = *reinterpret_cast<const float4*>(slot + ((jj * kLinLanes + r) * kDeltaCols + col) * 4);
+    st[jj * 4 + 0] = v4.x, st[jj * 4 + 1] = v4.y, st[jj * 4 + 2] = v4.z, st[jj * 4 + 3] = v4.w;
+  }
   const float head_decay = FORGET ? 0.f : decay[h];
-  // staging: 8 lanes per row copy the row's vectors (zeros beyond D and beyond the step's rows)
-  const int pt = tid >> 3, ps = tid & 7;
-  constexpr int PE = DP / 8;
-  float rq[PE], rk[PE], rv[kDeltaCols / 8];
+  // staging: kLinStage lanes per row copy the row's vectors (zeros beyond D and beyond the step's rows)
+  const int pt = tid / kLinStage, ps = tid % kLinStage;
+  constexpr int PE = DP / kLinStage;
+  float rq[PE], rk[PE], rv[kDeltaCols / kLinStage];
   auto fetch = [&](int c0) {
     const bool live = c0 + pt < n;
     const int64_t row = r0 + (live ? c0 + pt : 0);
     const float* p = proj + row * ld;
 #pragma unroll
     for (int m = 0; m < PE; ++m) {
-      const int i = ps + 8 * m;
+      const int i = ps + kLinStage * m;
       const bool ok = live && i < D;
       rq[m] = ok ? p[q_off + h * D + i] : 0.f;
       rk[m] = ok ? p[k_off + h * D + i] : 0.f;
     }
 #pragma unroll
-    for (int m = 0; m < kDeltaCols / 8; ++m) {
-      const int cc = cb * kDeltaCols + ps + 8 * m;
+    for (int m = 0; m < kDeltaCols / kLinStage; ++m) {
+      const int cc = cb * kDeltaCols + ps + kLinStage * m;
       rv[m] = (live && cc < Dv) ? p[v_off + h * Dv + cc] : 0.f;
     }
   };
@@ -1666,7 +1678,7 @@ __global__ __launch_bounds__(kDeltaThreads) void linear_attention_kernel(
     const bool live = c0 + pt < n;
 #pragma unroll
     for (int m = 0; m < PE; ++m) {
-      const int i = ps + 8 * m;
+      const int i = ps + kLinStage * m;
       const bool ok = live && i < D;
       qs[pt][i] = ok ? act(q_act, rq[m]) : 0.f;
       if constexpr (FORGET) {
@@ -1679,7 +1691,7 @@ __global__ __launch_bounds__(kDeltaThreads) void linear_attention_kernel(
       }
     }
 #pragma unroll
-    for (int m = 0; m < kDeltaCols / 8; ++m) vs[pt][ps + 8 * m] = act(v_act, rv[m]);
+    for (int m = 0; m < kDeltaCols / kLinStage; ++m) vs[pt][ps + kLinStage * m] = act(v_act, rv[m]);
     __syncthreads();
     if (c0 + kDeltaRows < n) fetch(c0 + kDeltaRows);
     const int nt = min(kDeltaRows, n - c0);
@@ -1691,9 +1703,9 @@ __global__ __launch_bounds__(kDeltaThreads) void linear_attention_kernel(
       float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
       for (int jj = 0; jj < DR / 4; ++jj) {
-        const float4 kv = k4[jj * 4 + r], qv = q4[jj * 4 + r];
+        const float4 kv = k4[jj * kLinLanes + r], qv = q4[jj * kLinLanes + r];
         float4 gv{head_decay, head_decay, head_decay, head_decay};
-        if constexpr (FORGET) gv = g4[jj * 4 + r];
+        if constexpr (FORGET) gv = g4[jj * kLinLanes + r];
         st[jj * 4 + 0] = fmaf(gv.x, st[jj * 4 + 0], kv.x * v);
         st[jj * 4 + 1] = fmaf(gv.y, st[jj * 4 + 1], kv.y * v);
         st[jj * 4 + 2] = fmaf(gv.z, st[jj * 4 + 2], kv.z * v);
@@ -1703,12 +1715,28 @@ __global__ __launch_bounds__(kDeltaThreads) void linear_attention_kernel(
         o2 = fmaf(st[jj * 4 + 2], qv.z, o2);
         o3 = fmaf(st[jj * 4 + 3], qv.w, o3);
       }
-      const float o = xor_sum<2>(xor_sum<1>((o0 + o1) + (o2 + o3)));
+      const float o = xor_sum<8>(xor_sum<4>(xor_sum<2>(xor_sum<1>((o0 + o1) + (o2 + o3)))));
       if (r == 0 && c < Dv) out[(int64_t)(r0 + c0 + t) * ldo + h * Dv + c] = o;
     }
   }
 #pragma unroll
-  for (int ii = 0; ii < DR; ++ii) slot[ii * kDeltaThreads + tid] = st[ii];
+  for (int jj = 0; jj < DR / 4; ++jj)
+    *reinterpret_cast<float4*>(slot + ((jj * kLinLanes + r) * kDeltaCols + col) * 4) =
+        float4{st[jj * 4 + 0], st[jj * 4 + 1], st[jj * 4 + 2], st[jj * 4 + 3]};
+}
+
+// out[row] <- out / rms(out over the row's `width` channels) * norm_w (* sigmoid(gate)): a workgroup per row, in place -
+// the read-out's norm over ALL heads of a row (delta_finish_kernel's wave per unit is for a norm per head)
+__global__ __launch_bounds__(256) void row_norm_gate_kernel(float* __restrict__ out, int64_t ldo,
+                                                            const float* __restrict__ gate_pre, int64_t ld_gate,
+                                                            const float* __restrict__ norm_w, int width, float eps) {
+  __shared__ float red[4];
+  float* o = out + (int64_t)blockIdx.x * ldo;
+  float sq = 0.f;
+  for (int d = threadIdx.x; d < width; d += 256) sq = fmaf(o[d], o[d], sq);
+  const float rstd = 1.f / sqrtf(block_sum256(sq, red) / (float)width + eps);
+  for (int d = threadIdx.x; d < width; d += 256)
+    o[d] = o[d] * rstd * norm_w[d] * (gate_pre ? sigmoid_f(gate_pre[(int64_t)blockIdx.x * ld_gate + d]) : 1.f);
 }
 
 }  // namespace mi
@@ -2100,10 +2128,13 @@ extern "C" int mi_gated_norm_add_f32(float* res, int64_t ldr, const float* y, in
   return check_launch();
 }
 
+// key channels per lane of linear_attention_kernel: the head's channels padded to 64, 128 or 256 over a column's lanes
+static int linear_dr(int D) { return D <= 64 ? 64 / kLinLanes : D <= 128 ? 128 / kLinLanes : D <= 256 ? 256 / kLinLanes : 0; }
+
 extern "C" int64_t mi_linear_attention_state_elems(int H, int D, int Dv) {
-  const int dr = delta_dr(D);
+  const int dr = linear_dr(D);
   if (!dr) return -1;
-  return (int64_t)H * ((Dv + kDeltaCols - 1) / kDeltaCols) * dr * kDeltaThreads;
+  return (int64_t)H * ((Dv + kDeltaCols - 1) / kDeltaCols) * dr * kLinThreads;
 }
 
 extern "C" int mi_linear_attention(const float* proj, int64_t ld, int q_off, int k_off, int v_off, int q_act, int k_act,
@@ -2118,30 +2149,33 @@ extern "C" int mi_linear_attention(const float* proj, int64_t ld, int q_off, int
   if (norm_w && norm_groups != 1 && norm_groups != H) return MI_EINVAL;
   for (int a : {q_act, k_act, v_act})
     if (a != MI_ACT_NONE && a != MI_ACT_SILU) return MI_EUNSUPPORTED;
-  const int dr = delta_dr(D);
+  const int dr = linear_dr(D);
   if (!dr || H > 65535) return MI_EUNSUPPORTED;
   if (n_rows == 0) return MI_OK;
   const dim3 grid(n_seqs, H, (Dv + kDeltaCols - 1) / kDeltaCols);
 #define MI_LINATTN(DR, KIND)                                                                                          \
-  hipLaunchKernelGGL((linear_attention_kernel<DR, KIND>), grid, dim3(kDeltaThreads), 0, S(stream), proj, ld, q_off,  \
+  hipLaunchKernelGGL((linear_attention_kernel<DR, KIND>), grid, dim3(kLinThreads), 0, S(stream), proj, ld, q_off,    \
                      k_off, v_off, q_act, k_act, v_act, decay, f_bias, lower, state, cu_q, kv_lens, slot_ids, H, D, Dv, \
                      out, ldo)
   if (decay_kind == MI_DECAY_HEAD) {
-    if (dr == 16) MI_LINATTN(16, MI_DECAY_HEAD);
-    else if (dr == 32) MI_LINATTN(32, MI_DECAY_HEAD);
-    else MI_LINATTN(64, MI_DECAY_HEAD);
+    if (dr == 64 / kLinLanes) MI_LINATTN(64 / kLinLanes, MI_DECAY_HEAD);
+    else if (dr == 128 / kLinLanes) MI_LINATTN(128 / kLinLanes, MI_DECAY_HEAD);
+    else MI_LINATTN(256 / kLinLanes, MI_DECAY_HEAD);
   } else {
-    if (dr == 16) MI_LINATTN(16, MI_DECAY_FORGET);
-    else if (dr == 32) MI_LINATTN(32, MI_DECAY_FORGET);
-    else MI_LINATTN(64, MI_DECAY_FORGET);
+    if (dr == 64 / kLinLanes) MI_LINATTN(64 / kLinLanes, MI_DECAY_FORGET);
+    else if (dr == 128 / kLinLanes) MI_LINATTN(128 / kLinLanes, MI_DECAY_FORGET);
+    else MI_LINATTN(256 / kLinLanes, MI_DECAY_FORGET);
   }
 #undef MI_LINATTN
   if (check_launch() != MI_OK) return MI_ELAUNCH;
   if (!norm_w) return MI_OK;
   // the read-out's norm: over each head's value channels (norm_groups == H, weight [Dv]) or over all heads' channels
   // together (norm_groups == 1, weight [H * Dv]); then the sigmoid gate, if any
-  const int groups = norm_groups, gw = norm_groups == 1 ? H * Dv : Dv;
-  hipLaunchKernelGGL(delta_finish_kernel, dim3((n_rows * groups + 3) / 4), dim3(256), 0, S(stream), out, ldo, gate_pre,
-                     ld_gate, norm_w, n_rows, groups, gw, eps);
+  if (norm_groups == 1 && H > 1)
+    hipLaunchKernelGGL(row_norm_gate_kernel, dim3(n_rows), dim3(256), 0, S(stream), out, ldo, gate_pre, ld_gate, norm_w,
+                       H * Dv, eps);
+  else
+    hipLaunchKernelGGL(delta_finish_kernel, dim3((n_rows * H + 3) / 4), dim3(256), 0, S(stream), out, ldo, gate_pre,
+                       ld_gate, norm_w, n_rows, H, Dv, eps);
   return check_launch();
 }
