@@ -750,8 +750,8 @@ int mi_gemm_any_batched(const float* x, int64_t ldx, int64_t x_batch, const void
 #define MI_BIAS_NONE  2
 /* mi_swa_attention with the bias named and the value rows ldv elements apart: v_cache may be k_cache itself with
  * ldv = D when a token's value is the first Dv channels of its key row (latent attention: G = 1).  window >= the longest
- * sequence: plain causal attention.  sink != NULL: every row's softmax denominator also holds exp(sink[h]), a logit per
- * head without key or value (not scaled, counted once).  workspace (may be NULL; workspace_elems floats): lets decode steps with few
+ * sequence: plain causal attention.  sink != NULL: every row's softmax normalises by sum_j exp(s_j) + exp(sink[h]) - a
+ * per-head logit used as it is, which only soaks up weight (no output term).  workspace (may be NULL; workspace_elems floats): lets decode steps with few
  * (row, kv head) units spread each unit's keys over several workgroups - rows * H * 2 k * (2 + Dv) floats allow k of
  * them, up to 16. */
 int mi_paged_attention_f32(const float* q, int64_t ldq, const void* k_cache, const void* v_cache, int64_t ldv,

@@ -21,6 +21,12 @@
 //   mi_route_grouped            router of a sparse feed-forward: softmax scores, additive choice correction, choice
 //                               restricted to the best groups of experts, top-k; weights = un-renormalised scores
 //   mi_moe_combine_f32          out[t] = sum_k w[t][k] * (identity expert ? h[t] : y[t * top_k + k])
+//   mi_causal_conv              the convolution with its activation and a "beside the identity" flag (y = x + conv(x))
+//   mi_gated_norm_add_f32       res += rms(y * sigmoid(gate)) * w, and the norm of the sum for the next sublayer
+//   mi_linear_attention         S <- diag(a_t) S + k_t v_t^T, o_t = S^T q_t with a decay per head or a forget gate per
+//                               key channel that also writes (k = 1 - f); read-out norm per head or over all heads, gate
+//   (further down: the pre-norm families' residual stack, minimal gated recurrence, latent and log-biased attention,
+//   plain top-k routing - each with its own header comment)
 //
 // Everything here is computed in fp32 (expf / logf / sqrtf of the device library, no fast-math), for both serving
 // dtypes: the bf16 mode differs only in the dtype of the WEIGHTS and of the K/V cache (and in the matrix-core attention
@@ -141,8 +147,9 @@ __global__ __launch_bounds__(256) void swa_prepare_kernel(float* __restrict__ pr
 // Distance bias of a score, taken off it: kind MI_BIAS_SLOPE: 2^(-8 (h + 1) / H) * dist (p1 == nullptr) or p1[h] * dist;
 // MI_BIAS_LOG: p1[h] * ln(1 + p2[h] * dist); MI_BIAS_NONE: nothing.  ldv: elements between two tokens' value rows (Dv,
 // or the key row's length when the values are the leading channels of the key rows of the same cache).
-// sink != nullptr: the softmax's denominator also holds exp(sink[h]) - a learned logit per head that has no key and no
-// value, is not scaled and counts once per row.
+// sink != nullptr: a row's softmax normalises by sum_j exp(s_j) + exp(sink[h]): the extra term is a learned per-head
+// logit taken as it is (the score scale does not touch it) that only soaks up weight - nothing is added to the output
+// for it.
 struct AttnBias {
   int kind;
   const float* p1;

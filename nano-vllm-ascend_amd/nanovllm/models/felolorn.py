@@ -1,7 +1,7 @@
 """Felolorn: a decoder whose layers - in an order its configuration lists - mix the sequence with a latent attention
 that knows no positions (queries through a latent of their own, a sink logit per head in the softmax), a linear
 attention whose state fades by a constant per head, or a linear attention whose forget gate also writes; each followed
-by a group-routed sparse feed-forward (or none).  Every sublayer is normed before AND after, reads - the mixers - its
+by a group-routed sparse feed-forward (or none).  Every sublayer sits between two RMS norms, reads - the mixers - its
 input through a short causal convolution beside the identity, and reaches the fp32 residual stream through a sigmoid
 gate computed from its own input:
 

@@ -84,8 +84,8 @@ def test_mechanism_alone(name, layers, kw, dtype):
 @pytest.mark.parametrize("shift", [0.0, -3.0])
 def test_router_choices_and_weights(T, n, top, count, keep, shift):
     """Sigmoid scores, the correction in the choice only, a group's value = its two best choice scores (a group of one: that
-    one), only the best groups eligible, un-renormalised weights; `shift`: all choice scores negative (an excluded expert
-    must count as minus infinity, not as 0); more outputs than a wave has lanes."""
+    one), only the best groups eligible, un-renormalised weights; `shift`: all choice scores negative (a dropped group's
+    experts must stay out even then: masking them with 0 would put them on top); more outputs than a wave has lanes."""
     from nanovllm import _C, ops
 
     g = torch.Generator().manual_seed(n + top)
