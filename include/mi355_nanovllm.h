@@ -691,6 +691,11 @@ int mi_causal_conv_silu(const float* x, int64_t ldx, const float* w, int taps, c
 int mi_causal_conv(const float* x, int64_t ldx, const float* w, int taps, const float* state, const int32_t* cu_q,
                    const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int rows, int channels, int silu,
                    int add_input, float* y, int64_t ldy, mi_stream stream);
+/* mi_causal_conv followed by mi_causal_conv_state; when no sequence of the step brings more than 8 rows
+ * (1 <= max_rows_per_seq <= 8: decode steps, short portions) both in one launch with the same arithmetic. */
+int mi_causal_conv_advance(const float* x, int64_t ldx, const float* w, int taps, float* state, const int32_t* cu_q,
+                           const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int rows, int max_rows_per_seq,
+                           int channels, int silu, int add_input, float* y, int64_t ldy, mi_stream stream);
 int mi_causal_conv_state(const float* x, int64_t ldx, int taps, float* state, const int32_t* cu_q,
                          const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int channels, mi_stream stream);
 /* Floats of recurrent state one sequence slot holds for mi_channel_delta (the kernel's own thread-order layout), or

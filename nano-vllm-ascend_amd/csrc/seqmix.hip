@@ -938,6 +938,54 @@ __global__ __launch_bounds__(256) void causal_conv_state_kernel(const float* __r
   for (int i = 0; i < L; ++i) st[(int64_t)i * C + c] = tail[i];
 }
 
+// Both in one launch for steps in which no sequence brings more than a few rows (decode steps, short portions): a thread
+// per (sequence, channel) keeps the tail in registers, walks its rows and writes the tail back - nothing else reads or
+// writes its entries, so there is no order to keep between launches.  The taps are summed in causal_conv_kernel's order.
+__global__ __launch_bounds__(256) void causal_conv_step_kernel(const float* __restrict__ x, int64_t ldx,
+                                                               const float* __restrict__ w, int taps,
+                                                               float* __restrict__ state,
+                                                               const int32_t* __restrict__ cu_q,
+                                                               const int32_t* __restrict__ kv_lens,
+                                                               const int32_t* __restrict__ slot_ids, int C, int silu,
+                                                               int add_input, float* __restrict__ y, int64_t ldy) {
+  const int s = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int r0 = cu_q[s], n = cu_q[s + 1] - r0;
+  if (n == 0) return;
+  const int start = kv_lens[s] - n;
+  const int L = taps - 1;
+  float* st = state + (int64_t)slot_ids[s] * L * C;
+  float tail[16], wt[17];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) tail[i] = (i < L && start > 0) ? st[(int64_t)i * C + c] : 0.f;
+#pragma unroll
+  for (int j = 0; j < 17; ++j) wt[j] = j < taps ? w[(int64_t)c * taps + j] : 0.f;
+  for (int r = 0; r < n; ++r) {
+    const float xr = x[(int64_t)(r0 + r) * ldx + c];
+    float acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+      if (j < L) acc = fmaf(wt[j], tail[j], acc);
+    float wl = 0.f;
+#pragma unroll
+    for (int j = 0; j < 17; ++j)
+      if (j == L) wl = wt[j];
+    acc = fmaf(wl, xr, acc);
+    if (silu) acc = acc / (1.f + expf(-acc));
+    if (add_input) acc += xr;
+    y[(int64_t)(r0 + r) * ldy + c] = acc;
+#pragma unroll
+    for (int i = 0; i < 15; ++i) tail[i] = i + 1 < L ? tail[i + 1] : tail[i];
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      if (i == L - 1) tail[i] = xr;
+  }
+#pragma unroll
+  for (int i = 0; i < 16; ++i)
+    if (i < L) st[(int64_t)i * C + c] = tail[i];
+}
+
 // ---------------------------------------------------------------------------------------------------------------
 // gated delta rule, decay per head and key channel
 // ---------------------------------------------------------------------------------------------------------------
@@ -1925,6 +1973,24 @@ extern "C" int mi_causal_conv(const float* x, int64_t ldx, const float* w, int t
   hipLaunchKernelGGL(causal_conv_kernel, dim3(rows, (channels + 255) / 256), dim3(256), 0, S(stream), x, ldx, w, taps,
                      state, cu_q, kv_lens, slot_ids, n_seqs, channels, silu, add_input, y, ldy);
   return check_launch();
+}
+
+extern "C" int mi_causal_conv_advance(const float* x, int64_t ldx, const float* w, int taps, float* state,
+                                      const int32_t* cu_q, const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs,
+                                      int rows, int max_rows_per_seq, int channels, int silu, int add_input, float* y,
+                                      int64_t ldy, mi_stream stream) {
+  if (!x || !w || !state || !cu_q || !kv_lens || !slot_ids || !y || rows < 0 || n_seqs < 1 || channels < 1) return MI_EINVAL;
+  if (taps < 1 || taps > 17 || n_seqs > 65535) return MI_EUNSUPPORTED;
+  if (rows == 0) return MI_OK;
+  if (max_rows_per_seq >= 1 && max_rows_per_seq <= 8) {
+    hipLaunchKernelGGL(causal_conv_step_kernel, dim3((channels + 255) / 256, n_seqs), dim3(256), 0, S(stream), x, ldx, w,
+                       taps, state, cu_q, kv_lens, slot_ids, channels, silu, add_input, y, ldy);
+    return check_launch();
+  }
+  const int rc = mi_causal_conv(x, ldx, w, taps, state, cu_q, kv_lens, slot_ids, n_seqs, rows, channels, silu, add_input, y,
+                                ldy, stream);
+  if (rc != MI_OK) return rc;
+  return mi_causal_conv_state(x, ldx, taps, state, cu_q, kv_lens, slot_ids, n_seqs, channels, stream);
 }
 
 extern "C" int mi_causal_conv_silu(const float* x, int64_t ldx, const float* w, int taps, const float* state,

@@ -180,6 +180,8 @@ _SIGNATURES = {
                                  c_int, c_int, c_int, c_float, _p, c_int64, _p, c_int64, _p]),
     "mi_causal_conv_silu": (c_int, [_p, c_int64, _p, c_int, _p, _p, _p, _p, c_int, c_int, c_int, _p, c_int64, _p]),
     "mi_causal_conv": (c_int, [_p, c_int64, _p, c_int, _p, _p, _p, _p, c_int, c_int, c_int, c_int, c_int, _p, c_int64, _p]),
+    "mi_causal_conv_advance": (c_int, [_p, c_int64, _p, c_int, _p, _p, _p, _p, c_int, c_int, c_int, c_int, c_int, c_int, _p,
+                                       c_int64, _p]),
     "mi_causal_conv_state": (c_int, [_p, c_int64, c_int, _p, _p, _p, _p, c_int, c_int, _p]),
     "mi_channel_delta_state_elems": (c_int64, [c_int, c_int, c_int]),
     "mi_channel_delta_workspace_elems": (c_int64, [c_int, c_int, c_int, c_int]),

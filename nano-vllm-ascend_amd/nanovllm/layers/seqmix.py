@@ -150,8 +150,7 @@ class ChannelDeltaMixer(nn.Module):
         ctx = get_context()
         cu, kv, slots = ctx.cu_seqlens_q, ctx.kv_lens, ctx.state_slots
         pre = self.qkv(x)
-        qkv = ops.causal_conv_silu(pre, self.conv.weight, self.conv_state, cu, kv, slots)
-        ops.causal_conv_state(pre, self.taps, self.conv_state, cu, kv, slots)
+        qkv = ops.causal_conv_advance(pre, self.conv.weight, self.conv_state, cu, kv, slots, ctx.max_seqlen_q, silu=True)
         low = self.low(x)
         decay_pre = ops.gemm_any(self.low.cols(low, "a1"), self.a2)
         gate_pre = ops.gemm_any(self.low.cols(low, "g1"), self.g2)
@@ -402,9 +401,7 @@ class InputConvolution(nn.Module):
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         ctx = get_context()
         cu, kv, slots = ctx.cu_seqlens_q, ctx.kv_lens, ctx.state_slots
-        u = ops.causal_conv(h, self.weight, self.state, cu, kv, slots, silu=False, add_input=True)
-        ops.causal_conv_state(h, self.taps, self.state, cu, kv, slots)
-        return u
+        return ops.causal_conv_advance(h, self.weight, self.state, cu, kv, slots, ctx.max_seqlen_q, silu=False, add_input=True)
 
 
 class GatedOutputNorm(nn.Module):

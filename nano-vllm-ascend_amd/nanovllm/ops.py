@@ -1060,6 +1060,23 @@ def causal_conv(x, w, state, cu_q, kv_lens, slot_ids, silu: bool = False, add_in
     return y
 
 
+def causal_conv_advance(x, w, state, cu_q, kv_lens, slot_ids, max_rows_per_seq: int, silu: bool = False,
+                        add_input: bool = False) -> torch.Tensor:
+    """causal_conv() and causal_conv_state() as one call: the convolution over the step's rows, then the tail advanced;
+    one launch when no sequence brings more than 8 rows (a decode step)."""
+    require_gpu(x, w, state)
+    _f32(x, w, state)
+    _i32(cu_q, kv_lens, slot_ids)
+    rows, C = x.shape
+    taps = w.shape[1]
+    assert w.shape[0] == C and w.is_contiguous() and state.is_contiguous() and state.shape[1:] == (max(taps - 1, 1), C)
+    y = torch.empty((rows, C), dtype=_F32, device=x.device)
+    check(lib.mi_causal_conv_advance(ptr(x), x.stride(0), ptr(w), taps, ptr(state), ptr(cu_q), ptr(kv_lens), ptr(slot_ids),
+                                     kv_lens.numel(), rows, int(max_rows_per_seq), C, int(silu), int(add_input), ptr(y), C,
+                                     stream()), "mi_causal_conv_advance")
+    return y
+
+
 def causal_conv_state(x, taps: int, state, cu_q, kv_lens, slot_ids) -> None:
     require_gpu(x, state)
     _f32(x, state)

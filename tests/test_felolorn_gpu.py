@@ -164,6 +164,36 @@ def test_input_convolution_with_a_carried_tail(taps):
         at = [a + n for a, n in zip(at, counts)]
 
 
+@pytest.mark.parametrize("taps", [1, 2, 4, 17])
+@pytest.mark.parametrize("silu", [False, True])
+def test_convolution_and_tail_in_one_call(taps, silu):
+    """The combined call over three steps: short rows only (one launch does both), a long portion among them (two
+    launches), short ones again - the tail handed on between the two forms; bit-equal to the two separate calls."""
+    from nanovllm import ops
+
+    g = torch.Generator().manual_seed(taps + 7)
+    C, steps = 45, ([3, 1, 8], [2, 40, 1], [1, 1, 5])
+    w = torch.randn(C, taps, generator=g)
+    full = [torch.randn(sum(st[i] for st in steps), C, generator=g) for i in range(3)]
+    conv = [F.input_conv(f.double(), w.double()) for f in full]
+    want = [(c * torch.sigmoid(c) if silu else c + f.double()) for c, f in zip(conv, full)]
+    state = torch.randn(5, max(taps - 1, 1), C, generator=g).cuda()
+    twin = state.clone()
+    slots = torch.tensor([3, 1, 4], dtype=torch.int32).cuda()
+    at = [0, 0, 0]
+    for counts in steps:
+        x = torch.cat([f[a:a + n] for f, a, n in zip(full, at, counts)]).cuda()
+        cu = torch.tensor([0] + list(torch.tensor(counts).cumsum(0)), dtype=torch.int32).cuda()
+        kv = torch.tensor([a + n for a, n in zip(at, counts)], dtype=torch.int32).cuda()
+        got = ops.causal_conv_advance(x, w.cuda(), state, cu, kv, slots, max(counts), silu=silu, add_input=not silu)
+        two = ops.causal_conv(x, w.cuda(), twin, cu, kv, slots, silu=silu, add_input=not silu)
+        ops.causal_conv_state(x, taps, twin, cu, kv, slots)
+        assert torch.equal(got, two) and torch.equal(state, twin)
+        ref = torch.cat([wn[a:a + n] for wn, a, n in zip(want, at, counts)])
+        assert (got.cpu().double() - ref).abs().max() <= 2e-5
+        at = [a + n for a, n in zip(at, counts)]
+
+
 @pytest.mark.parametrize("kind", ["head", "forget"])
 @pytest.mark.parametrize("H,D,Dv", [(3, 8, 12), (2, 20, 32), (1, 64, 70), (2, 100, 16), (1, 128, 40), (1, 200, 33), (1, 256, 32)])
 def test_linear_attention_walk(kind, H, D, Dv):
