@@ -310,6 +310,67 @@ def test_attention_with_a_sink(cache, H, D, Dv, alias):
     assert (got - torch.stack([want[m - 1] for m in lens])).abs().max() <= bar
 
 
+@pytest.mark.parametrize("gate", [False, True])
+def test_latent_attention_layer_with_every_option(gate):
+    """The layer class with a query latent AND a rotated key part AND a sink (and the output gate on or off) - a combination
+    no model file wires yet - against the mechanism written out: a prompt's portion behind 21 cached positions."""
+    from nanovllm.layers.seqmix import LatentAttention
+    from nanovllm.utils.context import reset_context, set_context
+    from oracle import zedirax as Z
+
+    g = torch.Generator().manual_seed(3 + gate)
+    W, H, D, R, Dv, C, Q, dims, base, scale, eps = 40, 3, 12, 8, 10, 24, 14, 6, 30.0, 0.2, 1e-5
+    T, bs = 50, 16
+    old_default = torch.get_default_dtype()
+    torch.set_default_dtype(torch.float32)
+    try:
+        mod = LatentAttention(W, H, D, R, Dv, C, dims, base, scale, eps, q_rank=Q, gate=gate, sink=True)
+    finally:
+        torch.set_default_dtype(old_default)
+    p = {"dq": torch.randn(Q, W, generator=g) * W ** -0.5, "dq.norm": 1 + torch.randn(Q, generator=g) * 0.1,
+         "uq": torch.randn(H * (D + R), Q, generator=g) * Q ** -0.5, "dkv": torch.randn(C + R, W, generator=g) * W ** -0.5,
+         "dkv.norm": 1 + torch.randn(C, generator=g) * 0.1, "uk": torch.randn(H * D, C, generator=g) * C ** -0.5,
+         "uv": torch.randn(H * Dv, C, generator=g) * C ** -0.5, "g": torch.randn(H * Dv, W, generator=g) * W ** -0.5,
+         "o": torch.randn(W, H * Dv, generator=g) * (H * Dv) ** -0.5, "sink": torch.randn(H, generator=g)}
+    for name in ("dq", "dkv") + (("g",) if gate else ()):
+        mod.qcg.weight.weight_loader(mod.qcg.weight, p[name], name)
+    mod.q_norm.data.copy_(p["dq.norm"]), mod.uq.data.copy_(p["uq"]), mod.c_norm.data.copy_(p["dkv.norm"])
+    mod.uk_t.weight_loader(mod.uk_t, p["uk"]), mod.uv.weight_loader(mod.uv, p["uv"])
+    mod.o.data.copy_(p["o"]), mod.sink.data.copy_(p["sink"])
+    mod = mod.cuda()
+    mod.cache = torch.zeros(mod.cache_shape(6, bs), dtype=torch.float32, device="cuda")
+    u = torch.randn(T, W, generator=g)
+    # the mechanism written out (float64)
+    d = {k: v.double() for k, v in p.items()}
+    ud, pos = u.double(), torch.arange(T)
+    cq = F.rms_norm(ud @ d["dq"].T, d["dq.norm"], eps)
+    q = (cq @ d["uq"].T).view(T, H, D + R)
+    dkv = ud @ d["dkv"].T
+    c = F.rms_norm(dkv[:, :C], d["dkv.norm"], eps)
+    r, q_rot = Z.rotate(dkv[:, C:], pos, dims, base), Z.rotate(q[..., D:], pos, dims, base)
+    k, v = (c @ d["uk"].T).view(T, H, D), (c @ d["uv"].T).view(T, H, Dv)
+    sc = (torch.einsum("ihd,jhd->hij", q[..., :D], k) + torch.einsum("ihd,jd->hij", q_rot, r)) * scale
+    sc = sc.masked_fill(pos.view(1, T) > pos.view(T, 1), float("-inf"))
+    pr = torch.softmax(torch.cat([sc, d["sink"].view(H, 1, 1).expand(H, T, 1)], -1), -1)[..., :T]
+    o = torch.einsum("hij,jhd->ihd", pr, v).reshape(T, H * Dv)
+    if gate:
+        o = o * torch.sigmoid(ud @ d["g"].T)
+    want = o @ d["o"].T
+    table = torch.tensor([[4, 1, 3, 0]], dtype=torch.int32).cuda()
+    got = []
+    for a, b in ((0, 21), (21, T)):                # 21 positions into the cache, then the portion behind them
+        posn = torch.arange(a, b)
+        slots = (table[0].cpu()[posn // bs] * bs + posn % bs).to(torch.int32).cuda()
+        set_context(True, cu_seqlens_q=torch.tensor([0, b - a], dtype=torch.int32).cuda(),
+                    kv_lens=torch.tensor([b], dtype=torch.int32).cuda(), slot_mapping=slots, block_tables=table, block_size=bs,
+                    state_slots=torch.zeros(1, dtype=torch.int32).cuda(), max_seqlen_q=b - a, max_seqlen_k=b)
+        try:
+            got.append(mod(u[a:b].cuda()).cpu().double())
+        finally:
+            reset_context()
+    assert rel_err(torch.cat(got), want) <= F32_BAR
+
+
 @pytest.mark.parametrize("M", [1, 6, 40, 600])
 @pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32])
 def test_capped_head_projection_and_scaled_embedding(M, wdtype):
