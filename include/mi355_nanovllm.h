@@ -734,6 +734,8 @@ int mi_moe_combine_f32(const float* y, const float* h, int64_t ldh, const int32_
 #define MI_ACT_GELU_ERF  3  /* 0.5 z (1 + erf(z / sqrt 2)) */
 #define MI_ACT_SIGMOID   4
 #define MI_ACT_SOFTCAP   5  /* alpha tanh(z / alpha): the epilogue's alpha is the cap (mi_gemm_any_act, no w2) */
+#define MI_ACT_CLAMPED_GLU 6 /* two weights: g = min(x w^T, limit), u = clamp(x w2^T, -limit, limit);
+                              * y = g sigmoid(1.702 g) (u + 1)  (mi_gemm_any_grouped_glu) */
 /* mi_gemm_any with an epilogue: v = x w^T + bias (bias may be NULL); w2 != NULL: y = alpha * act(v) * (x w2^T + bias2),
  * else y = alpha * act(v). */
 int mi_gemm_any_act(const float* x, int64_t ldx, const void* w, const void* w2, int w_dtype, const float* bias,
@@ -743,6 +745,13 @@ int mi_gemm_any_act(const float* x, int64_t ldx, const void* w, const void* w2, 
 int mi_gemm_any_grouped_act(const float* x, int64_t ldx, const int32_t* x_rows, const void* w, const void* w2, int w_dtype,
                             int act, const int32_t* group_offsets, int n_groups, int rows_per_group_max, float* y,
                             int64_t ldy, const int32_t* y_rows, int N, int K, int exact, mi_stream stream);
+/* mi_gemm_any_grouped_act with MI_ACT_CLAMPED_GLU's limit and a scale per row: the accumulators of sorted row m are
+ * multiplied by row_scale[row_scale_rows ? row_scale_rows[m] : m] first (row_scale may be NULL) - the row's input scaled,
+ * e.g. by a routing weight that multiplies an expert's input rather than its output. */
+int mi_gemm_any_grouped_glu(const float* x, int64_t ldx, const int32_t* x_rows, const void* w, const void* w2, int w_dtype,
+                            int act, float limit, const float* row_scale, const int32_t* row_scale_rows,
+                            const int32_t* group_offsets, int n_groups, int rows_per_group_max, float* y, int64_t ldy,
+                            const int32_t* y_rows, int N, int K, int exact, mi_stream stream);
 /* n_batch products over the same M rows: batch b: y + b*y_batch [M][N] (ldy) = (x + b*x_batch) [M][K] (ldx) . w[b]^T
  * (w = [n_batch][N][K]) - a projection per head of head-major rows.  gate != NULL: times
  * sigmoid((gate + b*gate_batch)[row][n]) (ldgate). */
@@ -765,9 +774,23 @@ int mi_paged_attention_f32(const float* q, int64_t ldq, const void* k_cache, con
                            int window, float scale, int bias_kind, const float* bias_p1, const float* bias_p2,
                            const float* sink, const float* gate, int64_t ldg, float* out, int64_t ldo, float* workspace,
                            int64_t workspace_elems, mi_stream stream);
+/* mi_paged_attention_f32 with two more score / value options.  softcap > 0: the scaled, biased score s becomes
+ * softcap * tanh(s / softcap) before the mask and the softmax.  value_heads (a divisor of G): the value cache has this many
+ * heads, [blocks][value_heads][block_size][.], query head h reads value head h / (H / value_heads) - with fewer, wider value
+ * heads than key heads (a token's value heads side by side in one row, v_cache possibly pointing at a column of it) every
+ * query head weighs the values of several key/value heads at once: out [rows][H][Dv] with Dv the width read. */
+int mi_paged_attention_ext(const float* q, int64_t ldq, const void* k_cache, const void* v_cache, int64_t ldv,
+                           int cache_dtype, const int32_t* block_tables, int table_cols, const int32_t* cu_q,
+                           const int32_t* kv_lens, int n_seqs, int rows, int H, int G, int D, int Dv, int block_size,
+                           int window, float scale, int bias_kind, const float* bias_p1, const float* bias_p2,
+                           const float* sink, float softcap, int value_heads, const float* gate, int64_t ldg, float* out,
+                           int64_t ldo, float* workspace, int64_t workspace_elems, mi_stream stream);
 /* res += mult * y (y may be NULL); w != NULL: out = res / sqrt(mean(res^2) + eps) * (w + shift) per row. */
 int mi_add_rmsnorm_f32(float* res, int64_t ldr, const float* y, int64_t ldy, float mult, const float* w, float shift,
                        float eps, float* out, int64_t ldo, int rows, int width, mi_stream stream);
+/* The same with a vector vec [width] (may be NULL) added to every row: res += mult * y + vec. */
+int mi_add_vec_rmsnorm_f32(float* res, int64_t ldr, const float* y, int64_t ldy, float mult, const float* vec, const float* w,
+                           float shift, float eps, float* out, int64_t ldo, int rows, int width, mi_stream stream);
 /* stack = slots [rows][width] of the layers' results, slot_stride floats apart.  Slot n-1 += mult * y (y may be NULL);
  * slot n = sum_{j<n} coef[j] * slot j; norm_w != NULL: h = slot n / rms * (norm_w + shift). */
 int mi_depth_mix_f32(float* stack, int64_t slot_stride, int n, const float* coef, const float* y, int64_t ldy, float mult,
@@ -798,7 +821,8 @@ int mi_latent_prepare(const float* proj, int64_t ld, const float* q, int64_t ldq
 /* ids = the top_k largest logits (descending; equal: lower index), weights = softmax over those.  n_outputs <= 512. */
 int mi_route_topk(const float* logits, int64_t ld, int n_tokens, int n_outputs, int top_k, int32_t* ids, float* weights,
                   mi_stream stream);
-/* out[t] = sum_k weights[t][k] * y[t * top_k + k] + sigmoid(shared_gate[t]) * shared[t] (shared may be NULL). */
+/* out[t] = sum_k weights[t][k] * y[t * top_k + k] + sigmoid(shared_gate[t]) * shared[t] (shared may be NULL; weights may be
+ * NULL: every weight 1). */
 int mi_moe_combine_shared(const float* y, const int32_t* ids, const float* weights, int n_tokens, int top_k, int width,
                           const float* shared, int64_t ld_shared, const float* shared_gate, int64_t ld_gate, float* out,
                           int64_t ldo, mi_stream stream);
@@ -825,6 +849,30 @@ int mi_linear_attention(const float* proj, int64_t ld, int q_off, int k_off, int
                         int64_t ld_gate, const float* norm_w, int norm_groups, float* state, const int32_t* cu_q,
                         const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int n_rows, int H, int D, int Dv,
                         float eps, float* out, int64_t ldo, mi_stream stream);
+
+/* Rotary positions on the projected heads of a step's rows, in place: H query heads [D] at q_off and G key heads [D] at
+ * k_off of every proj row.  Position of a row as in mi_paged_attention_f32 (cu_q, kv_lens); angle of pair i =
+ * pos * inv_freq[i] (fp32), cos and sin times amp; the first rot_dims channels of a head are rotated, pairs (2i, 2i+1)
+ * or (i, i + rot_dims/2): */
+#define MI_ROT_INTERLEAVED 0
+#define MI_ROT_HALVES      1
+/* unit_norm: then every head is divided by sqrt(mean(head^2) + eps); key heads times k_mult on top.  k_cache != NULL: the
+ * key heads go to the paged cache [blocks][G][block_size][D] instead of back in place; v_cache != NULL: the row's Gv value
+ * heads [Dv] at v_off are copied to [blocks][Gv][block_size][Dv]; slots [rows] (< 0: the row stores nothing). */
+int mi_rotary_store(float* proj, int64_t ld, int q_off, int k_off, int v_off, int H, int G, int D, int Gv, int Dv,
+                    int rot_dims, int layout, const float* inv_freq, float amp, int unit_norm, float eps, float k_mult,
+                    const int32_t* cu_q, const int32_t* kv_lens, int n_seqs, void* k_cache, void* v_cache, int cache_dtype,
+                    const int32_t* slots, int rows, int block_size, mi_stream stream);
+/* Mixing of the heads' softmax weights p'_h = sum_g talk[h][g] p_g, applied to read-outs: o [rows][H][n_chunk * Dv] holds
+ * every query head's weights applied to the values of the key/value heads [c0, c0 + n_chunk);
+ * out[row][h][:] = out_scale * sum_g talk[h][g] o[row][g][(h / (H / G) - c0) * Dv + :] for the heads whose key/value head is
+ * in the chunk (the others are left alone). */
+int mi_head_mix(const float* o, int64_t ldo_in, const float* talk, int rows, int H, int G, int Dv, int c0, int n_chunk,
+                float out_scale, float* out, int64_t ldo, mi_stream stream);
+/* out[row][h] <- out_scale * out / sqrt(mean over Dv + eps) (* norm_w [Dv] if not NULL) (* act(gate_pre[row][h]) if not
+ * NULL, gate_act = MI_ACT_SIGMOID or MI_ACT_SILU), in place: the per-head norm and gate of a recurrence's read-out. */
+int mi_head_norm_gate(float* out, int64_t ldo, const float* gate_pre, int64_t ld_gate, int gate_act, const float* norm_w,
+                      float out_scale, int rows, int H, int Dv, float eps, mi_stream stream);
 
 /* ---- host-side hashing (reference: engine/block_manager.py:38-44) --------- */
 /* xxh64 of `len` bytes with seed 0, optionally prefixed by the 8 little-endian

@@ -46,6 +46,11 @@ struct GemmAnyArgs {
   // batched form (group_offsets == nullptr, gridDim.z > 1): batch b multiplies the M rows at x + b * x_batch with
   // w[b] into y + b * y_batch (a per-head projection of head-major rows: the batch stride is a head's width)
   int64_t x_batch, y_batch, gate_batch;
+  // grouped form: sorted row m's accumulators are multiplied by row_scale[row_scale_rows ? row_scale_rows[m] : m] before
+  // anything else (= its x row scaled, without touching x: an expert whose routing weight goes into its INPUT)
+  const float* row_scale;
+  const int32_t* row_scale_rows;
+  float limit;  // MI_ACT_CLAMPED_GLU
 };
 
 template <typename TW>
@@ -68,11 +73,20 @@ __device__ __forceinline__ float act_f(int act, float z) {
 }
 // what every kernel does to an accumulator (pair) before it stores it
 template <bool DUAL>
-__device__ __forceinline__ float finish(const GemmAnyArgs& a, int64_t yrow, int n, float v, float v2) {
+__device__ __forceinline__ float finish(const GemmAnyArgs& a, int64_t m, int64_t yrow, int n, float v, float v2) {
+  if (a.row_scale) {
+    const float rs = a.row_scale[a.row_scale_rows ? a.row_scale_rows[m] : m];
+    v *= rs, v2 *= rs;
+  }
   if (a.bias) v += a.bias[n];
   if (DUAL) {
     if (a.bias2) v2 += a.bias2[n];
-    v = act_f(a.act, v) * v2;
+    if (a.act == MI_ACT_CLAMPED_GLU) {  // g sigmoid(1.702 g) (u + 1) with g capped from above, u clamped to +-limit
+      const float g = fminf(v, a.limit), u = fminf(fmaxf(v2, -a.limit), a.limit);
+      v = g / (1.f + expf(-1.702f * g)) * (u + 1.f);
+    } else {
+      v = act_f(a.act, v) * v2;
+    }
   } else {
     v = a.act == MI_ACT_SOFTCAP ? tanhf(v / a.alpha) : act_f(a.act, v);  // (times alpha below: alpha tanh(v / alpha))
   }
@@ -180,7 +194,7 @@ __global__ __launch_bounds__(256) void gemm_any_fma_kernel(GemmAnyArgs a) {
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx * 4 + j;
       if (n >= a.N) continue;
-      a.y[yrow * a.ldy + n] = finish<DUAL>(a, yrow, n, acc[0][i][j], acc[DUAL ? 1 : 0][i][j]);
+      a.y[yrow * a.ldy + n] = finish<DUAL>(a, m, yrow, n, acc[0][i][j], acc[DUAL ? 1 : 0][i][j]);
     }
   }
 }
@@ -312,7 +326,7 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(GemmAnyArgs a) {
       float v[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        v[r] = n + r < a.N ? finish<DUAL>(a, yrow, n + r, acc[0][i][j][r], acc[ND - 1][i][j][r]) : 0.f;
+        v[r] = n + r < a.N ? finish<DUAL>(a, m, yrow, n + r, acc[0][i][j][r], acc[ND - 1][i][j][r]) : 0.f;
       float* yp = a.y + yrow * a.ldy + n;
       if (n + 4 <= a.N && (a.ldy % 4 == 0) && dev_aligned16(a.y)) {
         *reinterpret_cast<float4*>(yp) = float4{v[0], v[1], v[2], v[3]};
@@ -414,7 +428,7 @@ __global__ __launch_bounds__(256) void gemm_any_skinny_kernel(GemmAnyArgs a) {
     for (int r = 0; r < 4; ++r) {
       const int n = n0 + (lane >> 4) * 4 + r;
       if (n >= a.N) continue;
-      a.y[yrow * a.ldy + n] = finish<DUAL>(a, yrow, n, acc[0][f][r], acc[DUAL ? 1 : 0][f][r]);
+      a.y[yrow * a.ldy + n] = finish<DUAL>(a, m, yrow, n, acc[0][f][r], acc[DUAL ? 1 : 0][f][r]);
     }
   }
 }
@@ -459,7 +473,7 @@ __global__ __launch_bounds__(256) void gemm_any_rows_kernel(GemmAnyArgs a) {
     const float v2 = DUAL ? wave_sum(acc[DUAL ? 1 : 0][r]) : 0.f;
     if (lane == 0 && xr[r] >= 0) {
       const int64_t yrow = a.y_rows ? a.y_rows[m0 + r] : m0 + r;
-      a.y[yrow * a.ldy + n] = finish<DUAL>(a, yrow, n, v, v2);
+      a.y[yrow * a.ldy + n] = finish<DUAL>(a, m0 + r, yrow, n, v, v2);
     }
   }
 }
@@ -539,7 +553,7 @@ extern "C" int mi_gemm_any_act(const float* x, int64_t ldx, const void* w, const
                                int exact, mi_stream stream) {
   if (!x || !w || !y || M < 0 || N < 0 || K < 1 || ldx < K || ldy < N || !act_ok(act) || (bias2 && !w2)) return MI_EINVAL;
   if (act == MI_ACT_SOFTCAP && (w2 || !(alpha > 0.f))) return MI_EINVAL;
-  GemmAnyArgs a{x, ldx, w, w2, y, ldy, M, N, K, alpha, nullptr, nullptr, nullptr, bias, bias2, act, nullptr, 0, 0, 0, 0};
+  GemmAnyArgs a{x, ldx, w, w2, y, ldy, M, N, K, alpha, nullptr, nullptr, nullptr, bias, bias2, act, nullptr, 0, 0, 0, 0, nullptr, nullptr, 0.f};
   return gemm_any_dispatch(a, w_dtype, 1, M, exact ? 1 : 0, S(stream));
 }
 
@@ -549,7 +563,7 @@ extern "C" int mi_gemm_any_batched(const float* x, int64_t ldx, int64_t x_batch,
   if (!x || !w || !y || n_batch < 1 || M < 0 || N < 0 || K < 1 || ldx < K || ldy < N) return MI_EINVAL;
   if (n_batch > 65535) return MI_EUNSUPPORTED;
   GemmAnyArgs a{x, ldx, w, nullptr, y, ldy, M, N, K, 1.0f, nullptr, nullptr, nullptr, nullptr, nullptr, MI_ACT_NONE,
-                gate, ldgate, x_batch, y_batch, gate_batch};
+                gate, ldgate, x_batch, y_batch, gate_batch, nullptr, nullptr, 0.f};
   return gemm_any_dispatch(a, w_dtype, n_batch, M, exact ? 1 : 0, S(stream));
 }
 
@@ -565,11 +579,23 @@ extern "C" int mi_gemm_any_grouped_act(const float* x, int64_t ldx, const int32_
                                        int w_dtype, int act, const int32_t* group_offsets, int n_groups,
                                        int rows_per_group_max, float* y, int64_t ldy, const int32_t* y_rows, int N, int K,
                                        int exact, mi_stream stream) {
-  if (!x || !w || !y || !group_offsets || n_groups < 1 || rows_per_group_max < 0 || N < 0 || K < 1 || !act_ok(act) ||
-      act == MI_ACT_SOFTCAP)
+  if (act == MI_ACT_CLAMPED_GLU) return MI_EINVAL;  // (needs its limit: mi_gemm_any_grouped_glu)
+  return mi_gemm_any_grouped_glu(x, ldx, x_rows, w, w2, w_dtype, act, 0.f, nullptr, nullptr, group_offsets, n_groups,
+                                 rows_per_group_max, y, ldy, y_rows, N, K, exact, stream);
+}
+
+extern "C" int mi_gemm_any_grouped_glu(const float* x, int64_t ldx, const int32_t* x_rows, const void* w, const void* w2,
+                                       int w_dtype, int act, float limit, const float* row_scale,
+                                       const int32_t* row_scale_rows, const int32_t* group_offsets, int n_groups,
+                                       int rows_per_group_max, float* y, int64_t ldy, const int32_t* y_rows, int N, int K,
+                                       int exact, mi_stream stream) {
+  if (!x || !w || !y || !group_offsets || n_groups < 1 || rows_per_group_max < 0 || N < 0 || K < 1 ||
+      !(act_ok(act) || act == MI_ACT_CLAMPED_GLU) || act == MI_ACT_SOFTCAP)
     return MI_EINVAL;
+  if (act == MI_ACT_CLAMPED_GLU && (!w2 || !(limit > 0.f))) return MI_EINVAL;
+  if (row_scale_rows && !row_scale) return MI_EINVAL;
   if (n_groups > 65535) return MI_EUNSUPPORTED;
   GemmAnyArgs a{x, ldx, w, w2, y, ldy, rows_per_group_max, N, K, 1.0f, group_offsets, x_rows, y_rows, nullptr, nullptr,
-                act, nullptr, 0, 0, 0, 0};
+                act, nullptr, 0, 0, 0, 0, row_scale, row_scale_rows, limit};
   return gemm_any_dispatch(a, w_dtype, n_groups, rows_per_group_max, exact ? 1 : 0, S(stream));
 }

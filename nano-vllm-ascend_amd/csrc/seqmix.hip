@@ -150,12 +150,22 @@ __global__ __launch_bounds__(256) void swa_prepare_kernel(float* __restrict__ pr
 // sink != nullptr: a row's softmax normalises by sum_j exp(s_j) + exp(sink[h]): the extra term is a learned per-head
 // logit taken as it is (the score scale does not touch it) that only soaks up weight - nothing is added to the output
 // for it.
+// softcap > 0: the scaled, biased score s becomes softcap * tanh(s / softcap) before the mask and the softmax.
+// value_heads: the value cache has this many heads (a divisor of the key heads G; query head h reads value head
+// h / (H / value_heads)) - fewer, wider value heads than key heads let every query head weigh the values of SEVERAL
+// key/value heads at once (value rows holding the heads side by side), which is what mixing the heads' softmax weights
+// afterwards needs.
 struct AttnBias {
   int kind;
   const float* p1;
   const float* p2;
   const float* sink;
+  float softcap;
+  int value_heads;
 };
+__device__ __forceinline__ float capped(const AttnBias& bias, float s) {
+  return bias.softcap > 0.f ? bias.softcap * tanhf(s / bias.softcap) : s;
+}
 // the denominator of a finished row: its keys' sum l (relative to the running maximum m) plus the head's sink
 __device__ __forceinline__ float with_sink(const AttnBias& bias, int h, float m, float l) {
   return bias.sink ? l + expf(bias.sink[h] - m) : l;
@@ -210,6 +220,7 @@ __global__ __launch_bounds__(256) void swa_attention_kernel(const float* __restr
   const int pos = kv_lens[s] - (cu_q[s + 1] - cu_q[s]) + (row - cu_q[s]);
   const int lo = max(0, pos - window + 1);
   const int g = h / (H / G);
+  const int Gv = bias.value_heads, gv = h / (H / Gv);
   const HeadBias hb = head_bias(bias, h, H);
   const int32_t* table = block_tables + (int64_t)s * table_cols;
   float m = -INFINITY, l = 0.f;
@@ -225,7 +236,7 @@ __global__ __launch_bounds__(256) void swa_attention_kernel(const float* __restr
       const TC* kr = k_cache + ((blk * G + g) * block_size + j % block_size) * D;
       float dot = 0.f;
       for (int d = 0; d < D; ++d) dot = fmaf(qs[d], ld_f<TC>(kr + d), dot);
-      sc = dot * scale - dist_bias(hb, pos - j);
+      sc = capped(bias, dot * scale - dist_bias(hb, pos - j));
     }
     const float m_new = fmaxf(m, wave_max(sc));
     const float p = j <= pos ? expf(sc - m_new) : 0.f;
@@ -240,7 +251,7 @@ __global__ __launch_bounds__(256) void swa_attention_kernel(const float* __restr
     for (int jj = 0; jj < n_keys; ++jj) {
       const int jk = j0 + jj;
       const int64_t blk = table[jk / block_size];
-      const TC* vr = v_cache + ((blk * G + g) * block_size + jk % block_size) * ldv;
+      const TC* vr = v_cache + ((blk * Gv + gv) * block_size + jk % block_size) * ldv;
       const float pj = ps[jj];
 #pragma unroll
       for (int i = 0; i < VPL; ++i) {
@@ -308,6 +319,7 @@ __global__ __launch_bounds__(256) void swa_attention_vec_kernel(const float* __r
   float* qs = smem + wave * RPW * (D + 64);
   float* ps = qs + RPW * D;
   const int g = h / (H / G);
+  const int Gv = bias.value_heads, gv = h / (H / Gv);
   const HeadBias hb = head_bias(bias, h, H);
   const int lpr = 1 << lpr_log2, kg = lane >> lpr_log2, cg = lane & (lpr - 1), kpp = 64 >> lpr_log2;
   const int group_end = min(rg * RPW + RPW, n_rows);
@@ -355,7 +367,7 @@ __global__ __launch_bounds__(256) void swa_attention_vec_kernel(const float* __r
       for (int r = 0; r < RPW; ++r) {
         const int pos = pos0 + r;
         const bool vis = r < nr && j <= pos && j > pos - window;
-        const float sc = vis ? dots[r] * scale - dist_bias(hb, pos - j) : -INFINITY;
+        const float sc = vis ? capped(bias, dots[r] * scale - dist_bias(hb, pos - j)) : -INFINITY;
         const float m_new = fmaxf(m[r], wave_max(sc));
         const float p = vis ? expf(sc - m_new) : 0.f;
         const float corr = m[r] == -INFINITY ? 0.f : expf(m[r] - m_new);
@@ -372,7 +384,7 @@ __global__ __launch_bounds__(256) void swa_attention_vec_kernel(const float* __r
           const int jk = j0 + jj;
           const int64_t blk = table[jk / block_size];
           float vv[VEC];
-          ld_vec<TC, VEC>(v_cache + ((blk * G + g) * block_size + jk % block_size) * ldv + cg * VEC, vv);
+          ld_vec<TC, VEC>(v_cache + ((blk * Gv + gv) * block_size + jk % block_size) * ldv + cg * VEC, vv);
 #pragma unroll
           for (int r = 0; r < RPW; ++r) {
             const float pj = ps[r * 64 + jj];
@@ -456,6 +468,7 @@ __global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __
   if (wid >= n_groups * H) return;
   const int rg = wid / H, h = wid % H;
   const int g = h / (H / G);
+  const int Gv = bias.value_heads, gv = h / (H / Gv);
   const HeadBias hb = head_bias(bias, h, H);
   const int qi = lane & 15, kg = lane >> 4;
   const int dk = D / 32, dvt = Dv / 16;
@@ -531,6 +544,10 @@ __global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __
 #pragma unroll
         for (int e = 0; e < 8; ++e) sc[e] -= hb.a * (float)dist[e];
       }
+      if (bias.softcap > 0.f) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sc[e] = bias.softcap * tanhf(sc[e] / bias.softcap);
+      }
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         sc[e] = vis[e] ? sc[e] : -INFINITY;
@@ -560,7 +577,7 @@ __global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int key = min(j0 + (e >> 2) * 16 + kg * 4 + (e & 3), hi_key);  // (beyond the last key: weight 0)
-        vrow[e] = v_cache + (int64_t)cache_row(table, key, G, g, block_size, bs_shift) * (int)ldv +
+        vrow[e] = v_cache + (int64_t)cache_row(table, key, Gv, gv, block_size, bs_shift) * (int)ldv +
                   (PAIR ? 2 * qi : qi);
       }
       if constexpr (PAIR) {
@@ -634,6 +651,7 @@ __global__ __launch_bounds__(256) void paged_attention_heads_mfma_kernel(
   __shared__ float part_ml[3][2][64];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int row = blockIdx.x, g = blockIdx.y;
+  const int Gv = bias.value_heads, gv = g / (G / Gv);
   const int hpg = H / G;
   const int split = blockIdx.z % n_split;                 // this workgroup's share of the rounds of keys
   const int h0 = g * hpg + (blockIdx.z / n_split) * 16;   // first head of this workgroup's columns
@@ -679,7 +697,7 @@ __global__ __launch_bounds__(256) void paged_attention_heads_mfma_kernel(
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const int key = min(j0 + (e >> 2) * 16 + kg * 4 + (e & 3), hi_key);  // (beyond the last key: weight 0)
-      vrow[e] = v_cache + (int64_t)cache_row(table, key, G, g, block_size, bs_shift) * (int)ldv +
+      vrow[e] = v_cache + (int64_t)cache_row(table, key, Gv, gv, block_size, bs_shift) * (int)ldv +
                 (PAIR ? 2 * qi : qi);
     }
     uint32_t vw[PAIR ? DVM / 2 : 1][8];
@@ -725,6 +743,10 @@ __global__ __launch_bounds__(256) void paged_attention_heads_mfma_kernel(
     } else {
 #pragma unroll
       for (int e = 0; e < 8; ++e) sc[e] -= hb.a * (float)dist[e];
+    }
+    if (bias.softcap > 0.f) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sc[e] = bias.softcap * tanhf(sc[e] / bias.softcap);
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -1127,11 +1149,12 @@ __global__ __launch_bounds__(kDeltaThreads) void channel_delta_kernel(const floa
   for (int ii = 0; ii < DR; ++ii) slot[ii * kDeltaThreads + tid] = st[ii];
 }
 
-// out[row][h] <- out / rms(out over Dv) * norm_w (* sigmoid(gate) with a gate): one wave per (row, head), in place
+// out[row][h] <- out_scale * out / rms(out over Dv) * norm_w (* act(gate) with a gate; norm_w may be nullptr: no weight;
+// gate_act: MI_ACT_SIGMOID or MI_ACT_SILU): one wave per (row, head), in place
 __global__ __launch_bounds__(256) void delta_finish_kernel(float* __restrict__ out, int64_t ldo,
                                                            const float* __restrict__ gate_pre, int64_t ld_gate,
                                                            const float* __restrict__ norm_w, int n_rows, int H, int Dv,
-                                                           float eps) {
+                                                           float eps, int gate_act, float out_scale) {
   const int lane = threadIdx.x & 63;
   const int wid = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (wid >= n_rows * H) return;
@@ -1139,9 +1162,16 @@ __global__ __launch_bounds__(256) void delta_finish_kernel(float* __restrict__ o
   float* o = out + (int64_t)row * ldo + h * Dv;
   float sq = 0.f;
   for (int d = lane; d < Dv; d += 64) sq = fmaf(o[d], o[d], sq);
-  const float rstd = 1.f / sqrtf(wave_sum(sq) / (float)Dv + eps);
-  for (int d = lane; d < Dv; d += 64)
-    o[d] = o[d] * rstd * norm_w[d] * (gate_pre ? sigmoid_f(gate_pre[(int64_t)row * ld_gate + h * Dv + d]) : 1.f);
+  const float rstd = out_scale / sqrtf(wave_sum(sq) / (float)Dv + eps);
+  for (int d = lane; d < Dv; d += 64) {
+    float v = o[d] * rstd;
+    if (norm_w) v *= norm_w[d];
+    if (gate_pre) {
+      const float z = gate_pre[(int64_t)row * ld_gate + h * Dv + d];
+      v *= gate_act == MI_ACT_SILU ? z * sigmoid_f(z) : sigmoid_f(z);
+    }
+    o[d] = v;
+  }
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -1284,10 +1314,12 @@ __global__ __launch_bounds__(256) void moe_combine_f32_kernel(const float* __res
 // ---------------------------------------------------------------------------------------------------------------
 // pre-norm residual streams: RMS norm, residual update, depth-weighted mixing of the layers' results
 // ---------------------------------------------------------------------------------------------------------------
-// One workgroup per row.  res += mult * y (y may be nullptr); w != nullptr: out = res / sqrt(mean(res^2) + eps) * (w + shift)
-// (shift 1: weights stored around zero).  res == out is allowed (a plain norm in place).
+// One workgroup per row.  res += mult * y + vec (y, vec may be nullptr; vec [width] is the same for every row);
+// w != nullptr: out = res / sqrt(mean(res^2) + eps) * (w + shift) (shift 1: weights stored around zero).  res == out is
+// allowed (a plain norm in place).
 __global__ __launch_bounds__(256) void add_rmsnorm_f32_kernel(float* __restrict__ res, int64_t ldr,
                                                               const float* __restrict__ y, int64_t ldy, float mult,
+                                                              const float* __restrict__ vec,
                                                               const float* __restrict__ w, float shift, float eps,
                                                               float* __restrict__ out, int64_t ldo, int width) {
   __shared__ float red[4];
@@ -1296,10 +1328,9 @@ __global__ __launch_bounds__(256) void add_rmsnorm_f32_kernel(float* __restrict_
   float sq = 0.f;
   for (int c = threadIdx.x; c < width; c += 256) {
     float v = r[c];
-    if (yr) {
-      v = fmaf(mult, yr[c], v);
-      r[c] = v;
-    }
+    if (yr) v = fmaf(mult, yr[c], v);
+    if (vec) v += vec[c];
+    if (yr || vec) r[c] = v;
     sq = fmaf(v, v, sq);
   }
   if (!w) return;
@@ -1593,7 +1624,8 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict
     if (i < n_mine) wts[(int64_t)t * top_k + my_slot[i]] = mine[i] / sum;
 }
 
-// out[t] = sum_k w[t][k] y[t * top_k + k] + sigmoid(shared_gate[t]) * shared[t]   (shared == nullptr: no shared part)
+// out[t] = sum_k w[t][k] y[t * top_k + k] + sigmoid(shared_gate[t]) * shared[t]   (shared == nullptr: no shared part;
+// wts == nullptr: every weight 1 - experts whose weight already went into their input)
 __global__ __launch_bounds__(256) void moe_combine_shared_kernel(const float* __restrict__ y, const int32_t* __restrict__ ids,
                                                                  const float* __restrict__ wts, int top_k, int width,
                                                                  const float* __restrict__ shared, int64_t lds_,
@@ -1603,7 +1635,8 @@ __global__ __launch_bounds__(256) void moe_combine_shared_kernel(const float* __
   const float sgate = shared ? sigmoid_f(shared_gate[(int64_t)t * ldsg]) : 0.f;
   for (int c = threadIdx.x; c < width; c += 256) {
     float acc = 0.f;
-    for (int k = 0; k < top_k; ++k) acc = fmaf(wts[(int64_t)t * top_k + k], y[((int64_t)t * top_k + k) * width + c], acc);
+    for (int k = 0; k < top_k; ++k)
+      acc = fmaf(wts ? wts[(int64_t)t * top_k + k] : 1.f, y[((int64_t)t * top_k + k) * width + c], acc);
     if (shared) acc = fmaf(sgate, shared[(int64_t)t * lds_ + c], acc);
     out[(int64_t)t * ldo + c] = acc;
   }
@@ -1794,6 +1827,95 @@ __global__ __launch_bounds__(256) void row_norm_gate_kernel(float* __restrict__ 
     o[d] = o[d] * rstd * norm_w[d] * (gate_pre ? sigmoid_f(gate_pre[(int64_t)blockIdx.x * ld_gate + d]) : 1.f);
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// rotary positions on projected heads, unit norm per head, K / V rows to the pages
+// ---------------------------------------------------------------------------------------------------------------
+// One workgroup per step row, a wave per head in turn (H query heads at q_off, G key heads at k_off of the row).  The
+// first rot_dims channels of a head are rotated by the angles pos * inv_freq[i] (fp32 product, sincosf), cos and sin
+// times `amp`: channel pairs (2i, 2i + 1) (layout MI_ROT_INTERLEAVED) or (i, i + rot_dims / 2) (MI_ROT_HALVES).  Then,
+// unit_norm: the head is divided by sqrt(mean(head^2) + eps); key heads are multiplied by k_mult on top.  Query heads
+// are written back in place.  Key heads go to the paged cache [blocks][G][block_size][D] when k_cache != nullptr (rows
+// with slot < 0 store nothing), else back in place.  v_cache != nullptr: the row's Gv value heads of Dv channels at v_off
+// are copied to [blocks][Gv][block_size][Dv] as they are.
+template <typename TC>
+__global__ __launch_bounds__(256) void rotary_store_kernel(float* __restrict__ proj, int64_t ld, int q_off, int k_off,
+                                                           int v_off, int H, int G, int D, int Gv, int Dv, int rot_dims,
+                                                           int layout, const float* __restrict__ inv_freq, float amp,
+                                                           int unit_norm, float eps, float k_mult,
+                                                           const int32_t* __restrict__ cu_q,
+                                                           const int32_t* __restrict__ kv_lens, int n_seqs,
+                                                           TC* __restrict__ k_cache, TC* __restrict__ v_cache,
+                                                           const int32_t* __restrict__ slots, int block_size) {
+  extern __shared__ float smem[];  // per wave: one head [D]
+  const int row = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int s = seq_of_row(cu_q, n_seqs, row);
+  const float pos = (float)(kv_lens[s] - (cu_q[s + 1] - cu_q[s]) + (row - cu_q[s]));
+  const int slot = slots ? slots[row] : -1;
+  const int64_t blk = slot >= 0 ? slot / block_size : 0;
+  const int off = slot >= 0 ? slot % block_size : 0;
+  float* hv = smem + wave * D;
+  float* base = proj + (int64_t)row * ld;
+  const int half = rot_dims / 2;
+  for (int head = wave; head < H + G; head += 4) {
+    const bool is_k = head >= H;
+    float* src = base + (is_k ? k_off + (head - H) * D : q_off + head * D);
+    for (int d = lane; d < D; d += 64) hv[d] = src[d];
+    __builtin_amdgcn_wave_barrier();
+    for (int i = lane; i < half; i += 64) {
+      float sn, cs;
+      sincosf(pos * inv_freq[i], &sn, &cs);
+      sn *= amp, cs *= amp;
+      const int ia = layout == MI_ROT_INTERLEAVED ? 2 * i : i, ib = layout == MI_ROT_INTERLEAVED ? 2 * i + 1 : i + half;
+      const float a = hv[ia], b = hv[ib];
+      hv[ia] = a * cs - b * sn;
+      hv[ib] = b * cs + a * sn;
+    }
+    __builtin_amdgcn_wave_barrier();
+    float mult = is_k ? k_mult : 1.f;
+    if (unit_norm) {
+      float sq = 0.f;
+      for (int d = lane; d < D; d += 64) sq = fmaf(hv[d], hv[d], sq);
+      mult *= 1.f / sqrtf(wave_sum(sq) / (float)D + eps);
+    }
+    if (is_k && k_cache) {
+      if (slot >= 0) {
+        TC* dst = k_cache + ((blk * G + (head - H)) * block_size + off) * D;
+        for (int d = lane; d < D; d += 64) st_f<TC>(dst + d, hv[d] * mult);
+      }
+    } else {
+      for (int d = lane; d < D; d += 64) src[d] = hv[d] * mult;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (v_cache && slot >= 0) {
+    const float* v = base + v_off;
+    for (int c = threadIdx.x; c < Gv * Dv; c += 256) {
+      const int g = c / Dv, d = c - g * Dv;
+      st_f<TC>(v_cache + ((blk * Gv + g) * block_size + off) * Dv + d, v[c]);
+    }
+  }
+}
+
+// Mixing of the heads' softmax weights, done on the read-outs (the mixing is linear in the weights): `o` holds, for every
+// query head g, that head's weights applied to the values of n_chunk key/value heads [c0, c0 + n_chunk) side by side
+// ([rows][H][n_chunk * Dv]); out[row][h][:] = out_scale * sum_g talk[h][g] * o[row][g][(kv(h) - c0) * Dv + :] for the heads
+// h whose own key/value head kv(h) = h / (H / G) lies in the chunk.  A thread per (row, h, d).
+__global__ __launch_bounds__(256) void head_mix_kernel(const float* __restrict__ o, int64_t ldo_in,
+                                                       const float* __restrict__ talk, int n_rows, int H, int G, int Dv,
+                                                       int c0, int n_chunk, float out_scale, float* __restrict__ out,
+                                                       int64_t ldo) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)n_rows * H * Dv) return;
+  const int d = (int)(idx % Dv), h = (int)((idx / Dv) % H);
+  const int64_t row = idx / ((int64_t)Dv * H);
+  const int c = h / (H / G) - c0;
+  if (c < 0 || c >= n_chunk) return;
+  const float* src = o + row * ldo_in + c * Dv + d;
+  float acc = 0.f;
+  for (int g = 0; g < H; ++g) acc = fmaf(talk[h * H + g], src[(int64_t)g * n_chunk * Dv], acc);
+  out[row * ldo + h * Dv + d] = acc * out_scale;
+}
+
 }  // namespace mi
 
 using namespace mi;
@@ -1848,9 +1970,11 @@ static int launch_swa(const float* q, int64_t ldq, const void* kc, const void* v
   const TC* k = static_cast<const TC*>(kc);
   const TC* v = static_cast<const TC*>(vc);
   constexpr int VEC = 16 / sizeof(TC);
+  // (v may point at a column of wider value rows: the fast forms load it in 16-byte / 4-byte pieces)
+  const bool v16 = (reinterpret_cast<uintptr_t>(vc) & 15u) == 0;
   if constexpr (sizeof(TC) == 2) {
     // prompt portions over a bf16 cache: the matrix-core form
-    if (rows > n_seqs && D % 32 == 0 && Dv % 16 == 0 && D <= 256 && Dv <= 256 && ldv % 2 == 0) {
+    if (v16 && rows > n_seqs && D % 32 == 0 && Dv % 16 == 0 && D <= 256 && Dv <= 256 && ldv % 2 == 0) {
       const dim3 grid_m((((rows + 15) / 16) * H + 3) / 4);
 #define MI_SWA_MFMA(DKM, DVM, PAIR)                                                                                    \
   hipLaunchKernelGGL((swa_attention_mfma_kernel<DKM, DVM, PAIR>), grid_m, dim3(256), 0, st, q, ldq, k, v, bt, cols, cu_q, \
@@ -1866,7 +1990,7 @@ static int launch_swa(const float* q, int64_t ldq, const void* kc, const void* v
   }
   if constexpr (sizeof(TC) == 2) {
     // decode steps (a row per sequence) over a bf16 cache: the matrix-core form with a kv head's query heads as columns
-    if (rows == n_seqs && D % 32 == 0 && Dv % 16 == 0 && D <= 256 && Dv <= 256 && ldv % 2 == 0 && G <= 65535) {
+    if (v16 && rows == n_seqs && D % 32 == 0 && Dv % 16 == 0 && D <= 256 && Dv <= 256 && ldv % 2 == 0 && G <= 65535) {
       // few (row, kv head) units: up to 16 workgroups share one, each taking every n_split-th batch of four rounds, and
       // a second launch merges their partial results (workspace: rows * H * n_split * (2 + Dv) floats)
       const int chunks = (H / G + 15) / 16;
@@ -1898,7 +2022,7 @@ static int launch_swa(const float* q, int64_t ldq, const void* kc, const void* v
       return check_launch();
     }
   }
-  if (D % VEC == 0 && Dv % VEC == 0 && Dv / VEC <= 64 && ldv % VEC == 0) {
+  if (v16 && D % VEC == 0 && Dv % VEC == 0 && Dv / VEC <= 64 && ldv % VEC == 0) {
     int lpr_log2 = 0;
     while ((1 << lpr_log2) * VEC < Dv) ++lpr_log2;
     // rows == n_seqs: every sequence brings one row (a decode step): a wave per row; else four rows per wave
@@ -1946,13 +2070,26 @@ extern "C" int mi_paged_attention_f32(const float* q, int64_t ldq, const void* k
                                       const float* bias_p2, const float* sink, const float* gate, int64_t ldg,
                                       float* out, int64_t ldo, float* workspace, int64_t workspace_elems,
                                       mi_stream stream) {
+  return mi_paged_attention_ext(q, ldq, k_cache, v_cache, ldv, cache_dtype, block_tables, table_cols, cu_q, kv_lens, n_seqs,
+                                rows, H, G, D, Dv, block_size, window, scale, bias_kind, bias_p1, bias_p2, sink, 0.f, G,
+                                gate, ldg, out, ldo, workspace, workspace_elems, stream);
+}
+
+extern "C" int mi_paged_attention_ext(const float* q, int64_t ldq, const void* k_cache, const void* v_cache, int64_t ldv,
+                                      int cache_dtype, const int32_t* block_tables, int table_cols, const int32_t* cu_q,
+                                      const int32_t* kv_lens, int n_seqs, int rows, int H, int G, int D, int Dv,
+                                      int block_size, int window, float scale, int bias_kind, const float* bias_p1,
+                                      const float* bias_p2, const float* sink, float softcap, int value_heads,
+                                      const float* gate, int64_t ldg, float* out, int64_t ldo, float* workspace,
+                                      int64_t workspace_elems, mi_stream stream) {
   if (!q || !k_cache || !v_cache || !block_tables || !cu_q || !kv_lens || !out || rows < 0 || n_seqs < 1) return MI_EINVAL;
   if (H < 1 || G < 1 || H % G || D < 1 || Dv < 1 || block_size < 1 || window < 1 || table_cols < 1 || ldv < Dv) return MI_EINVAL;
+  if (value_heads < 1 || G % value_heads || !(softcap >= 0.f)) return MI_EINVAL;
   if (bias_kind != MI_BIAS_SLOPE && bias_kind != MI_BIAS_LOG && bias_kind != MI_BIAS_NONE) return MI_EINVAL;
   if (bias_kind == MI_BIAS_LOG && (!bias_p1 || !bias_p2)) return MI_EINVAL;
   if (Dv > 512 || D > 4096) return MI_EUNSUPPORTED;
   if (rows == 0) return MI_OK;
-  const AttnBias bias{bias_kind, bias_p1, bias_p2, sink};
+  const AttnBias bias{bias_kind, bias_p1, bias_p2, sink, softcap, value_heads};
   if (cache_dtype == MI_DTYPE_BF16)
     return launch_swa<uint16_t>(q, ldq, k_cache, v_cache, block_tables, table_cols, cu_q, kv_lens, n_seqs, rows, H, G, D,
                                 Dv, block_size, window, scale, bias, ldv, gate, ldg, out, ldo, workspace, workspace_elems,
@@ -2049,7 +2186,7 @@ extern "C" int mi_channel_delta(const float* qkv, int64_t ld, int q_off, int k_o
 #undef MI_DELTA
   if (check_launch() != MI_OK) return MI_ELAUNCH;
   hipLaunchKernelGGL(delta_finish_kernel, dim3((n_rows * H + 3) / 4), dim3(256), 0, S(stream), out, ldo, gate_pre,
-                     ld_gate, norm_w, n_rows, H, Dv, eps);
+                     ld_gate, norm_w, n_rows, H, Dv, eps, MI_ACT_SIGMOID, 1.f);
   return check_launch();
 }
 
@@ -2081,10 +2218,16 @@ extern "C" int mi_moe_combine_f32(const float* y, const float* h, int64_t ldh, c
 
 extern "C" int mi_add_rmsnorm_f32(float* res, int64_t ldr, const float* y, int64_t ldy, float mult, const float* w,
                                   float shift, float eps, float* out, int64_t ldo, int rows, int width, mi_stream stream) {
+  return mi_add_vec_rmsnorm_f32(res, ldr, y, ldy, mult, nullptr, w, shift, eps, out, ldo, rows, width, stream);
+}
+
+extern "C" int mi_add_vec_rmsnorm_f32(float* res, int64_t ldr, const float* y, int64_t ldy, float mult, const float* vec,
+                                      const float* w, float shift, float eps, float* out, int64_t ldo, int rows, int width,
+                                      mi_stream stream) {
   if (!res || rows < 0 || width < 1 || ldr < width || (y && ldy < width) || (w && (!out || ldo < width))) return MI_EINVAL;
-  if (rows == 0 || (!y && !w)) return MI_OK;
-  hipLaunchKernelGGL(add_rmsnorm_f32_kernel, dim3(rows), dim3(256), 0, S(stream), res, ldr, y, ldy, mult, w, shift, eps, out,
-                     ldo, width);
+  if (rows == 0 || (!y && !w && !vec)) return MI_OK;
+  hipLaunchKernelGGL(add_rmsnorm_f32_kernel, dim3(rows), dim3(256), 0, S(stream), res, ldr, y, ldy, mult, vec, w, shift,
+                     eps, out, ldo, width);
   return check_launch();
 }
 
@@ -2184,7 +2327,7 @@ extern "C" int mi_route_topk(const float* logits, int64_t ld, int n_tokens, int 
 extern "C" int mi_moe_combine_shared(const float* y, const int32_t* ids, const float* weights, int n_tokens, int top_k,
                                      int width, const float* shared, int64_t ld_shared, const float* shared_gate,
                                      int64_t ld_gate, float* out, int64_t ldo, mi_stream stream) {
-  if (!y || !ids || !weights || !out || n_tokens < 0 || top_k < 1 || width < 1 || (shared && !shared_gate)) return MI_EINVAL;
+  if (!y || !ids || !out || n_tokens < 0 || top_k < 1 || width < 1 || (shared && !shared_gate)) return MI_EINVAL;
   if (n_tokens == 0) return MI_OK;
   hipLaunchKernelGGL(moe_combine_shared_kernel, dim3(n_tokens), dim3(256), 0, S(stream), y, ids, weights, top_k, width,
                      shared, ld_shared, shared_gate, ld_gate, out, ldo);
@@ -2249,6 +2392,56 @@ extern "C" int mi_linear_attention(const float* proj, int64_t ld, int q_off, int
                        H * Dv, eps);
   else
     hipLaunchKernelGGL(delta_finish_kernel, dim3((n_rows * H + 3) / 4), dim3(256), 0, S(stream), out, ldo, gate_pre,
-                       ld_gate, norm_w, n_rows, H, Dv, eps);
+                       ld_gate, norm_w, n_rows, H, Dv, eps, MI_ACT_SIGMOID, 1.f);
+  return check_launch();
+}
+
+extern "C" int mi_rotary_store(float* proj, int64_t ld, int q_off, int k_off, int v_off, int H, int G, int D, int Gv, int Dv,
+                               int rot_dims, int layout, const float* inv_freq, float amp, int unit_norm, float eps,
+                               float k_mult, const int32_t* cu_q, const int32_t* kv_lens, int n_seqs, void* k_cache,
+                               void* v_cache, int cache_dtype, const int32_t* slots, int rows, int block_size,
+                               mi_stream stream) {
+  if (!proj || !cu_q || !kv_lens || rows < 0 || n_seqs < 1 || H < 0 || G < 0 || D < 1 || block_size < 1) return MI_EINVAL;
+  if (rot_dims < 0 || rot_dims > D || rot_dims % 2 || (rot_dims && !inv_freq)) return MI_EINVAL;
+  if (layout != MI_ROT_INTERLEAVED && layout != MI_ROT_HALVES) return MI_EINVAL;
+  if ((k_cache || v_cache) && !slots) return MI_EINVAL;
+  if (v_cache && (Gv < 1 || Dv < 1)) return MI_EINVAL;
+  if (q_off + (int64_t)H * D > ld || k_off + (int64_t)G * D > ld || (v_cache && v_off + (int64_t)Gv * Dv > ld)) return MI_EINVAL;
+  const size_t lds = 4 * (size_t)D * sizeof(float);
+  if (lds > 48 * 1024) return MI_EUNSUPPORTED;
+  if (rows == 0) return MI_OK;
+  if (cache_dtype == MI_DTYPE_BF16)
+    hipLaunchKernelGGL(rotary_store_kernel<uint16_t>, dim3(rows), dim3(256), lds, S(stream), proj, ld, q_off, k_off, v_off,
+                       H, G, D, Gv, Dv, rot_dims, layout, inv_freq, amp, unit_norm, eps, k_mult, cu_q, kv_lens, n_seqs,
+                       static_cast<uint16_t*>(k_cache), static_cast<uint16_t*>(v_cache), slots, block_size);
+  else if (cache_dtype == MI_DTYPE_F32)
+    hipLaunchKernelGGL(rotary_store_kernel<float>, dim3(rows), dim3(256), lds, S(stream), proj, ld, q_off, k_off, v_off, H,
+                       G, D, Gv, Dv, rot_dims, layout, inv_freq, amp, unit_norm, eps, k_mult, cu_q, kv_lens, n_seqs,
+                       static_cast<float*>(k_cache), static_cast<float*>(v_cache), slots, block_size);
+  else
+    return MI_EINVAL;
+  return check_launch();
+}
+
+extern "C" int mi_head_mix(const float* o, int64_t ldo_in, const float* talk, int rows, int H, int G, int Dv, int c0,
+                           int n_chunk, float out_scale, float* out, int64_t ldo, mi_stream stream) {
+  if (!o || !talk || !out || rows < 0 || H < 1 || G < 1 || H % G || Dv < 1 || c0 < 0 || n_chunk < 1 || c0 + n_chunk > G)
+    return MI_EINVAL;
+  if (ldo_in < (int64_t)H * n_chunk * Dv || ldo < (int64_t)H * Dv) return MI_EINVAL;
+  if (rows == 0) return MI_OK;
+  const int64_t n = (int64_t)rows * H * Dv;
+  hipLaunchKernelGGL(head_mix_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, S(stream), o, ldo_in, talk, rows, H,
+                     G, Dv, c0, n_chunk, out_scale, out, ldo);
+  return check_launch();
+}
+
+extern "C" int mi_head_norm_gate(float* out, int64_t ldo, const float* gate_pre, int64_t ld_gate, int gate_act,
+                                 const float* norm_w, float out_scale, int rows, int H, int Dv, float eps,
+                                 mi_stream stream) {
+  if (!out || rows < 0 || H < 1 || Dv < 1 || ldo < (int64_t)H * Dv || (gate_pre && ld_gate < (int64_t)H * Dv)) return MI_EINVAL;
+  if (gate_act != MI_ACT_SIGMOID && gate_act != MI_ACT_SILU) return MI_EINVAL;
+  if (rows == 0) return MI_OK;
+  hipLaunchKernelGGL(delta_finish_kernel, dim3((rows * H + 3) / 4), dim3(256), 0, S(stream), out, ldo, gate_pre, ld_gate,
+                     norm_w, rows, H, Dv, eps, gate_act, out_scale);
   return check_launch();
 }

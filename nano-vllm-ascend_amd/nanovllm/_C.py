@@ -25,7 +25,8 @@ LIB_PATH = os.environ.get(
 MI_OK = 0
 MI_EUNSUPPORTED = -2
 DTYPE_BF16, DTYPE_F32 = 0, 1
-ACT_NONE, ACT_SILU, ACT_GELU_TANH, ACT_GELU_ERF, ACT_SIGMOID, ACT_SOFTCAP = range(6)   # MI_ACT_*
+ACT_NONE, ACT_SILU, ACT_GELU_TANH, ACT_GELU_ERF, ACT_SIGMOID, ACT_SOFTCAP, ACT_CLAMPED_GLU = range(7)   # MI_ACT_*
+ROT_INTERLEAVED, ROT_HALVES = range(2)                                    # MI_ROT_*
 ROUTE_SOFTMAX, ROUTE_SIGMOID = range(2)                                   # MI_ROUTE_*
 ROUTE_GROUP_MAX, ROUTE_GROUP_TOP2 = range(2)                              # MI_ROUTE_GROUP_*
 DECAY_HEAD, DECAY_FORGET = range(2)                                       # MI_DECAY_*
@@ -214,6 +215,17 @@ _SIGNATURES = {
     "mi_linear_attention_state_elems": (c_int64, [c_int, c_int, c_int]),
     "mi_linear_attention": (c_int, [_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _p, _p, _p, _p, c_int64,
                                     _p, c_int, _p, _p, _p, _p, c_int, c_int, c_int, c_int, c_int, c_float, _p, c_int64, _p]),
+    "mi_paged_attention_ext": (c_int, [_p, c_int64, _p, _p, c_int64, c_int, _p, c_int, _p, _p, c_int, c_int, c_int, c_int,
+                                       c_int, c_int, c_int, c_int, c_float, c_int, _p, _p, _p, c_float, c_int, _p, c_int64,
+                                       _p, c_int64, _p, c_int64, _p]),
+    "mi_add_vec_rmsnorm_f32": (c_int, [_p, c_int64, _p, c_int64, c_float, _p, _p, c_float, c_float, _p, c_int64, c_int, c_int,
+                                       _p]),
+    "mi_gemm_any_grouped_glu": (c_int, [_p, c_int64, _p, _p, _p, c_int, c_int, c_float, _p, _p, _p, c_int, c_int, _p, c_int64,
+                                        _p, c_int, c_int, c_int, _p]),
+    "mi_rotary_store": (c_int, [_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _p, c_float,
+                                c_int, c_float, c_float, _p, _p, c_int, _p, _p, c_int, _p, c_int, c_int, _p]),
+    "mi_head_mix": (c_int, [_p, c_int64, _p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _p, c_int64, _p]),
+    "mi_head_norm_gate": (c_int, [_p, c_int64, _p, c_int64, c_int, _p, c_float, c_int, c_int, c_int, c_float, _p]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

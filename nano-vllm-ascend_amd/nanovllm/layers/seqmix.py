@@ -26,6 +26,21 @@ configuration:
                             residual; the same launch norms the sum for the next sublayer
   HeadDecayLinearAttention  linear attention with a matrix state per head that fades by one constant per head
   ForgetGateLinearAttention linear attention whose per-channel forget gate f also writes: S <- diag(f) S + (1 - f) v^T
+  rotary_table              rotation frequencies of a head's channel pairs, optionally rescaled for long contexts (a ramp
+                            between the fast pairs, kept, and the slow ones, divided by a factor; cos / sin amplified)
+  RotaryWindowAttention     paged sliding-window attention over rotated (interleaved pairs) queries and keys, optionally
+                            behind short causal convolutions, with unit-normed heads, a sink logit per head, capped scores
+                            and mixing of the heads' softmax weights as options
+  Retention                 linear attention over rotated (half-split pairs) queries and keys with a fixed decay per head,
+                            per-head unit norm and a SiLU gate on the read-out
+  SinkAttentionMixer        projections + RotaryWindowAttention + output projection
+  ParallelMixers            a RotaryWindowAttention and a Retention side by side on the same input: one merged input
+                            projection, one merged output projection of the two scaled read-outs
+  InputWeightedSparseMLP    top-k experts by sigmoid score whose weight multiplies the expert's INPUT; experts
+                            W_d (g sigmoid(1.702 g) (u + 1)) with g capped and u clamped
+
+Layers whose weights a model runs several times per step (a looped stack) keep one cache / state per pass ("lane"): their
+forward takes the lane's number.
 
 Activations are fp32 tensors [rows, features]; matrices are stored in the serving dtype (bf16, or fp32 for the exact
 mode), vectors always in fp32.  A step's rows come with the metadata of utils/context.py: cu_seqlens_q, kv_lens (the
@@ -472,3 +487,207 @@ class ForgetGateLinearAttention(_LinearAttentionState):
                                  _C.DECAY_FORGET, None, self.f_bias, self.lower, None, self.norm, self.H, self.state,
                                  ctx.cu_seqlens_q, ctx.kv_lens, ctx.state_slots, self.H, self.D, self.Dv, self.eps)
         return ops.gemm_any(o, self.o)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# looped pre-norm families: rotated window attention with its options, retention, experts weighted on their input
+# ---------------------------------------------------------------------------------------------------------------------
+def rotary_table(dims: int, base: float, scaling: dict | None = None):
+    """-> (frequencies [dims / 2] fp32, amplitude of cos and sin).  f_i = base^(-2 i / dims), computed in double and
+    rounded once.  scaling {factor, original, fast, slow}: with c(r) = dims ln(original / (2 pi r)) / (2 ln base) - the pair
+    that turns r times over `original` positions - the pairs up to floor c(fast) keep their frequency, those from
+    ceil c(slow) on are divided by `factor`, a linear ramp in between; cos and sin are multiplied by 0.1 ln(factor) + 1."""
+    import math
+
+    f = [float(base) ** (-2.0 * i / dims) for i in range(dims // 2)]
+    amp = 1.0
+    if scaling:
+        factor, original = float(scaling["factor"]), float(scaling["original"])
+
+        def c(r):
+            return dims * math.log(original / (2 * math.pi * r)) / (2 * math.log(float(base)))
+
+        lo = max(math.floor(c(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(c(float(scaling["slow"]))), dims - 1)
+        ramp = [min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0) for i in range(dims // 2)]
+        f = [fi / factor * r + fi * (1 - r) for fi, r in zip(f, ramp)]
+        amp = 0.1 * math.log(factor) + 1.0
+    return torch.tensor(f or [0.0], dtype=torch.float64).to(torch.float32), amp
+
+
+class RotaryWindowAttention(nn.Module):
+    """The attention itself, on projections its owner made (`parts`: name -> rows of the q / k / v projections, to be laid
+    out next to each other in this order).  conv_taps > 0: q, k and v first pass a causal convolution per channel (filters
+    `conv.weight` [channels, taps], no activation), whose last taps - 1 inputs are the sequence's state.  Then q and k are
+    rotated (pairs 2i, 2i + 1 of the first rot_dims channels), unit_norm: each head divided by its root mean square;
+    s = scale q.k, softcap > 0: s <- softcap tanh(s / softcap); keys 0 <= i - j < window; softmax, sink: with
+    exp(sink_h) in the denominator; talk: the heads' weights are mixed, p'_h = sum_g talk[h, g] p_g, before head h applies
+    them to the values of its own key/value head.
+
+    The mixing is linear in the weights, so it is done on read-outs: every query head's weights are applied to the values
+    of ALL key/value heads (the value pages hold a token's heads side by side as ONE wide head, read in chunks of at most
+    256 channels), then out_h = sum_g talk[h, g] o[g, kv(h)]."""
+
+    def __init__(self, heads: int, kv_heads: int, dim: int, vdim: int, window: int, scale: float, eps: float,
+                 rot_dims: int, rot_base: float, rot_scaling: dict | None = None, unit_norm: bool = False,
+                 sink: bool = False, softcap: float = 0.0, conv_taps: int = 0, talk: bool = False):
+        super().__init__()
+        assert heads % kv_heads == 0 and 0 <= rot_dims <= dim and rot_dims % 2 == 0
+        self.H, self.G, self.D, self.Dv = heads, kv_heads, dim, vdim
+        self.window, self.scale, self.eps, self.unit_norm, self.softcap = window, scale, eps, unit_norm, softcap
+        self.rot_dims = rot_dims
+        freq, self.rot_amp = rotary_table(rot_dims, rot_base, rot_scaling) if rot_dims else (torch.zeros(1), 1.0)
+        self.register_buffer("inv_freq", freq, persistent=False)
+        self.parts = {"q": heads * dim, "k": kv_heads * dim, "v": kv_heads * vdim}
+        self.sink = _vector(heads) if sink else None
+        self.talk = nn.Parameter(torch.eye(heads, dtype=torch.float32), requires_grad=False) if talk else None
+        self.conv = MergedRows(conv_taps, self.parts, dtype=torch.float32) if conv_taps else None
+        self.k_cache, self.v_cache, self.conv_state = [], [], []   # one per lane
+        # value heads read together by one launch when the weights are mixed
+        self.chunk = max(1, min(kv_heads, 256 // vdim)) if talk else 0
+
+    @property
+    def out_features(self) -> int:
+        return self.H * self.Dv
+
+    def cache_shapes(self, num_blocks: int, block_size: int):
+        v = (num_blocks, 1, block_size, self.G * self.Dv) if self.talk is not None else (num_blocks, self.G, block_size, self.Dv)
+        return (num_blocks, self.G, block_size, self.D), v
+
+    def conv_state_shape(self, n_slots: int):
+        return (n_slots, max(self.conv.weight.shape[1] - 1, 1), self.conv.weight.shape[0]) if self.conv is not None else None
+
+    def attend(self, y: torch.Tensor, q_off: int, lane: int, out: torch.Tensor, out_scale: float = 1.0) -> None:
+        """y: rows holding q | k | v from column q_off on; out [rows, >= heads * vdim] receives out_scale * read-out."""
+        ctx = get_context()
+        H, G, D, Dv = self.H, self.G, self.D, self.Dv
+        n = H * D + G * D + G * Dv
+        if self.conv is not None:
+            y = ops.causal_conv_advance(y[:, q_off:q_off + n], self.conv.weight, self.conv_state[lane], ctx.cu_seqlens_q,
+                                        ctx.kv_lens, ctx.state_slots, ctx.max_seqlen_q)
+            q_off = 0
+        k_off, v_off = q_off + H * D, q_off + H * D + G * D
+        kc, vc = self.k_cache[lane], self.v_cache[lane]
+        ops.rotary_store(y, q_off, k_off, v_off, H, G, D, self.rot_dims, _C.ROT_INTERLEAVED, self.inv_freq, self.rot_amp,
+                         self.unit_norm, self.eps, 1.0, ctx.cu_seqlens_q, ctx.kv_lens, kc, vc, ctx.slot_mapping, ctx.block_size)
+        q = y[:, q_off:q_off + H * D]
+        if self.talk is None:
+            ops.paged_attention_f32(q, kc, vc, Dv, ctx.block_tables, ctx.cu_seqlens_q, ctx.kv_lens, H, G, D, Dv,
+                                    ctx.block_size, self.window, self.scale, _C.BIAS_NONE, sink=self.sink,
+                                    softcap=self.softcap, out=out)
+            if out_scale != 1.0:
+                out.mul_(out_scale)
+            return
+        for c0 in range(0, G, self.chunk):
+            nc = min(self.chunk, G - c0)
+            o = ops.paged_attention_f32(q, kc, vc, G * Dv, ctx.block_tables, ctx.cu_seqlens_q, ctx.kv_lens, H, G, D, nc * Dv,
+                                        ctx.block_size, self.window, self.scale, _C.BIAS_NONE, sink=self.sink,
+                                        softcap=self.softcap, value_heads=1, v_offset=c0 * Dv)
+            ops.head_mix(o, self.talk, H, G, Dv, c0, nc, out, out_scale)
+
+
+class Retention(nn.Module):
+    """q, k rotated (pairs i, i + rot_dims / 2 of the first rot_dims channels), k <- k dim^(-1/2); per head
+    S <- decay_h S + k v^T, o = S^T q (fp32 state per sequence slot and lane, no softmax, no denominator); each head's o
+    divided by its root mean square, times silu(g)."""
+
+    def __init__(self, heads: int, dim: int, vdim: int, decay, eps: float, rot_dims: int, rot_base: float,
+                 rot_scaling: dict | None = None):
+        super().__init__()
+        assert len(decay) == heads and 0 <= rot_dims <= dim and rot_dims % 2 == 0
+        self.H, self.D, self.Dv, self.eps, self.rot_dims = heads, dim, vdim, eps, rot_dims
+        freq, self.rot_amp = rotary_table(rot_dims, rot_base, rot_scaling) if rot_dims else (torch.zeros(1), 1.0)
+        self.register_buffer("inv_freq", freq, persistent=False)
+        self.register_buffer("decay", torch.tensor([float(d) for d in decay], dtype=torch.float64).to(torch.float32),
+                             persistent=False)
+        self.parts = {"q": heads * dim, "k": heads * dim, "v": heads * vdim, "g": heads * vdim}
+        self.state = []   # one per lane
+
+    @property
+    def out_features(self) -> int:
+        return self.H * self.Dv
+
+    def state_shape(self, n_slots: int):
+        return (n_slots, ops.linear_attention_state_elems(self.H, self.D, self.Dv))
+
+    def scan(self, y: torch.Tensor, q_off: int, lane: int, out: torch.Tensor, out_scale: float = 1.0) -> None:
+        """y: rows holding q | k | v | g from column q_off on (q and k are rotated in place); out [rows, heads * vdim]."""
+        ctx = get_context()
+        H, D, Dv = self.H, self.D, self.Dv
+        k_off, v_off, g_off = q_off + H * D, q_off + 2 * H * D, q_off + 2 * H * D + H * Dv
+        ops.rotary_store(y, q_off, k_off, v_off, H, H, D, self.rot_dims, _C.ROT_HALVES, self.inv_freq, self.rot_amp, False,
+                         self.eps, D ** -0.5, ctx.cu_seqlens_q, ctx.kv_lens)
+        ops.linear_attention(y, q_off, k_off, v_off, (_C.ACT_NONE,) * 3, _C.DECAY_HEAD, self.decay, None, None, None, None, H,
+                             self.state[lane], ctx.cu_seqlens_q, ctx.kv_lens, ctx.state_slots, H, D, Dv, self.eps, out=out)
+        ops.head_norm_gate(out, y[:, g_off:g_off + H * Dv], _C.ACT_SILU, None, H, Dv, self.eps, out_scale)
+
+
+class SinkAttentionMixer(nn.Module):
+    """W_o attention(W_q h, W_k h, W_v h) with a RotaryWindowAttention as the attention."""
+
+    def __init__(self, width: int, attention: RotaryWindowAttention):
+        super().__init__()
+        self.attn = attention
+        self.qkv = MergedRows(width, attention.parts)
+        self.o = _matrix(width, attention.out_features)
+
+    def forward(self, h: torch.Tensor, lane: int = 0) -> torch.Tensor:
+        y = self.qkv(h)
+        out = torch.empty((h.shape[0], self.attn.out_features), dtype=torch.float32, device=h.device)
+        self.attn.attend(y, 0, lane, out)
+        return ops.gemm_any(out, self.o)
+
+
+class ParallelMixers(nn.Module):
+    """left_scale * W_ol attention(h) + right_scale * W_or retention(h): the seven projections of h are ONE product, the
+    two read-outs are written, already scaled, side by side into one buffer, and [W_ol | W_or] is ONE output projection."""
+
+    def __init__(self, width: int, left: RotaryWindowAttention, right: Retention, left_scale: float, right_scale: float):
+        super().__init__()
+        self.left, self.right, self.left_scale, self.right_scale = left, right, left_scale, right_scale
+        parts = {f"left.{n}": r for n, r in left.parts.items()}
+        parts.update({f"right.{n}": r for n, r in right.parts.items()})
+        self.proj = MergedRows(width, parts)
+        nl, nr = left.out_features, right.out_features
+        self.o = _matrix(width, nl + nr)
+        spans = {"left": (0, nl), "right": (nl, nr)}
+
+        def load_o(param, tensor, side):
+            off, n = spans[side]
+            assert tensor.shape[1] == n, (side, tuple(tensor.shape), n)
+            param.data[:, off:off + n].copy_(tensor)
+        self.o.weight_loader = load_o
+
+    def forward(self, h: torch.Tensor, lane: int = 0) -> torch.Tensor:
+        y = self.proj(h)
+        nl, nr = self.left.out_features, self.right.out_features
+        out = torch.empty((h.shape[0], nl + nr), dtype=torch.float32, device=h.device)
+        self.left.attend(y, self.proj.offsets["left.q"][0], lane, out[:, :nl], self.left_scale)
+        self.right.scan(y, self.proj.offsets["right.q"][0], lane, out[:, nl:], self.right_scale)
+        return ops.gemm_any(out, self.o)
+
+
+class InputWeightedSparseMLP(nn.Module):
+    """Router logits in true 32-bit, scores = sigmoid; the top_k largest; out = sum_k expert_k(s_k h) - the score
+    multiplies the expert's input (experts have no biases: s (W h) = W (s h), so it is applied to the first projections'
+    accumulators).  Expert: g = min(W_g x, limit), u = clamp(W_u x, -limit, limit), W_d (g sigmoid(1.702 g) (u + 1))."""
+
+    def __init__(self, width: int, ff: int, experts: int, top_k: int, limit: float):
+        super().__init__()
+        assert 1 <= top_k <= experts and limit > 0
+        self.E, self.top_k, self.limit = experts, top_k, limit
+        self.router = _matrix(experts, width)
+        self.register_buffer("no_correction", torch.zeros(experts, dtype=torch.float32), persistent=False)
+        self.gate, self.up, self.down = _matrix(experts, ff, width), _matrix(experts, ff, width), _matrix(experts, width, ff)
+        for p in (self.gate, self.up, self.down):
+            p.weight_loader = lambda param, tensor, expert: param.data[expert].copy_(tensor)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        z = ops.gemm_any(h, self.router, exact=True)
+        ids, wts = ops.route_grouped(z, self.no_correction, self.top_k, 1, 1, _C.ROUTE_SIGMOID, _C.ROUTE_GROUP_MAX)
+        offsets, pair_token, pair_index = ops.moe_sort(ids, self.E)
+        P = ids.numel()
+        a = ops.gemm_any_grouped_glu(h, pair_token, self.gate, self.up, _C.ACT_CLAMPED_GLU, self.limit, wts, pair_index,
+                                     offsets, P, None, P)
+        y = ops.gemm_any_grouped(a, None, self.down, None, offsets, P, pair_index, P)
+        return ops.moe_combine_shared(y, ids, None, h.shape[1])

@@ -7,6 +7,7 @@ from nanovllm.models.gazutar import GazutarConfig, GazutarForCausalLM
 from nanovllm.models.llama import LlamaForCausalLM
 from nanovllm.models.qwen3 import Qwen3ForCausalLM
 from nanovllm.models.qwen3_moe import Qwen3MoeForCausalLM
+from nanovllm.models.sanevik import SanevikConfig, SanevikForCausalLM
 from nanovllm.models.zedirax import ZediraxConfig, ZediraxForCausalLM
 
 model_dict = {
@@ -17,6 +18,7 @@ model_dict = {
     "Gazutar": GazutarForCausalLM,
     "Zedirax": ZediraxForCausalLM,
     "Felolorn": FelolornForCausalLM,
+    "Sanevik": SanevikForCausalLM,
 }
 
 # designs whose config.json is not a transformers configuration: {"architecture": <name>, ...} -> the reader of it
@@ -24,6 +26,7 @@ native_configs = {
     "Gazutar": GazutarConfig,
     "Zedirax": ZediraxConfig,
     "Felolorn": FelolornConfig,
+    "Sanevik": SanevikConfig,
 }
 
 

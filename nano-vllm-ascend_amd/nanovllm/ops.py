@@ -1203,44 +1203,53 @@ def gemm_any_batched(x, x_batch: int, w, out, out_batch: int, gate=None, gate_ba
 
 def paged_attention_f32(q, k_cache, v_cache, ldv: int, block_tables, cu_q, kv_lens, H: int, G: int, D: int, Dv: int,
                         block_size: int, window: int, scale: float, bias_kind: int = _C.BIAS_NONE, bias_p1=None, bias_p2=None,
-                        gate=None, sink=None) -> torch.Tensor:
-    """Paged causal attention over fp32 queries; see mi_paged_attention_f32 (bias kinds, values inside the key rows, a
-    sink logit per head in the softmax's denominator)."""
+                        gate=None, sink=None, softcap: float = 0.0, value_heads: int | None = None,
+                        v_offset: int = 0, out=None) -> torch.Tensor:
+    """Paged causal attention over fp32 queries; see mi_paged_attention_ext (bias kinds, values inside the key rows, a
+    sink logit per head in the softmax's denominator, capped scores, fewer and wider value heads than key heads with the
+    value rows read from column v_offset on)."""
     require_gpu(q, k_cache, v_cache, block_tables, cu_q, kv_lens)
     _f32(q, gate, bias_p1, bias_p2, sink)
     assert sink is None or (sink.numel() == H and sink.is_contiguous())
     _i32(block_tables, cu_q, kv_lens)
     rows, n_seqs = q.shape[0], kv_lens.numel()
     assert q.shape[1] >= H * D and cu_q.numel() == n_seqs + 1 and block_tables.shape[0] >= n_seqs
-    assert k_cache.dtype == v_cache.dtype
+    assert k_cache.dtype == v_cache.dtype and 0 <= v_offset and v_offset + Dv <= ldv
     assert bias_kind != _C.BIAS_LOG or (bias_p1.numel() == H and bias_p2.numel() == H)
-    out = torch.empty((rows, H * Dv), dtype=_F32, device=q.device)
+    if out is None:
+        out = torch.empty((rows, H * Dv), dtype=_F32, device=q.device)
+    _f32(out)
+    assert out.shape[0] == rows and out.shape[1] >= H * Dv   # (a column slice of a wider buffer is fine)
     ws = None
     if rows == n_seqs and k_cache.dtype == _BF16:   # a decode step: room for up to 16 workgroups per (row, head)
         ws = torch.empty(rows * H * 32 * (2 + Dv), dtype=_F32, device=q.device)
-    check(lib.mi_paged_attention_f32(ptr(q), q.stride(0), ptr(k_cache), ptr(v_cache), int(ldv), _dt(k_cache),
+    check(lib.mi_paged_attention_ext(ptr(q), q.stride(0), ptr(k_cache), ptr(v_cache) + v_offset * v_cache.element_size(),
+                                     int(ldv), _dt(k_cache),
                                      ptr(block_tables), block_tables.shape[1], ptr(cu_q), ptr(kv_lens), n_seqs, rows, H, G,
                                      D, Dv, block_size, int(min(window, 2 ** 31 - 1)), float(scale), int(bias_kind),
-                                     ptr(bias_p1), ptr(bias_p2), ptr(sink), ptr(gate),
+                                     ptr(bias_p1), ptr(bias_p2), ptr(sink), float(softcap),
+                                     int(G if value_heads is None else value_heads), ptr(gate),
                                      gate.stride(0) if gate is not None else 0,
                                      ptr(out), out.stride(0), ptr(ws), ws.numel() if ws is not None else 0, stream()),
-          "mi_paged_attention_f32")
+          "mi_paged_attention_ext")
     return out
 
 
-def add_rmsnorm_f32(res, y, mult: float, w, eps: float, shift: float = 0.0, out=None):
-    """res += mult * y in place (y None: unchanged); w given: returns res / rms(res) * (w + shift), else None."""
+def add_rmsnorm_f32(res, y, mult: float, w, eps: float, shift: float = 0.0, out=None, vec=None):
+    """res += mult * y + vec in place (y / vec None: nothing added; vec [width] goes to every row); w given: returns
+    res / rms(res) * (w + shift), else None."""
     require_gpu(res)
-    _f32(res, y, w, out)
+    _f32(res, y, w, out, vec)
     rows, width = res.shape
     assert y is None or y.shape == res.shape
+    assert vec is None or (vec.numel() == width and vec.is_contiguous())
     if w is not None:
         assert w.numel() == width
         if out is None:
             out = torch.empty((rows, width), dtype=_F32, device=res.device)
-    check(lib.mi_add_rmsnorm_f32(ptr(res), res.stride(0), ptr(y), y.stride(0) if y is not None else 0, float(mult), ptr(w),
-                                 float(shift), float(eps), ptr(out), out.stride(0) if out is not None else 0, rows, width,
-                                 stream()), "mi_add_rmsnorm_f32")
+    check(lib.mi_add_vec_rmsnorm_f32(ptr(res), res.stride(0), ptr(y), y.stride(0) if y is not None else 0, float(mult),
+                                     ptr(vec), ptr(w), float(shift), float(eps), ptr(out),
+                                     out.stride(0) if out is not None else 0, rows, width, stream()), "mi_add_vec_rmsnorm_f32")
     return out
 
 
@@ -1320,8 +1329,8 @@ def route_topk(logits, n_outputs: int, top_k: int):
 
 
 def moe_combine_shared(y, ids, wts, width: int, shared=None, shared_gate=None) -> torch.Tensor:
-    """sum_k wts[t][k] * y[t * top_k + k] (+ sigmoid(shared_gate[t]) * shared[t])."""
-    require_gpu(y, ids, wts)
+    """sum_k wts[t][k] * y[t * top_k + k] (+ sigmoid(shared_gate[t]) * shared[t]); wts None: every weight 1."""
+    require_gpu(y, ids)
     _f32(y, wts, shared)
     T, top_k = ids.shape
     assert y.shape == (T * top_k, width) and y.is_contiguous()
@@ -1362,7 +1371,8 @@ def linear_attention_state_elems(H: int, D: int, Dv: int) -> int:
 
 
 def linear_attention(proj, q_off: int, k_off: int, v_off: int, acts, decay_kind: int, decay, f_bias, lower, gate_pre, norm_w,
-                     norm_groups: int, state, cu_q, kv_lens, slot_ids, H: int, D: int, Dv: int, eps: float) -> torch.Tensor:
+                     norm_groups: int, state, cu_q, kv_lens, slot_ids, H: int, D: int, Dv: int, eps: float,
+                     out=None) -> torch.Tensor:
     """S <- diag(a) S + k v^T, o = S^T q per head over the step's rows (see mi_linear_attention); acts = the (q, k, v)
     activations; returns the normed (and gated) read-out [rows, H * Dv]."""
     require_gpu(proj, state)
@@ -1377,10 +1387,82 @@ def linear_attention(proj, q_off: int, k_off: int, v_off: int, acts, decay_kind:
         assert f_bias.numel() == H * D and lower.numel() == H * D
     assert norm_w is None or norm_w.numel() == (H * Dv if norm_groups == 1 else Dv)
     assert gate_pre is None or (gate_pre.shape[0] == rows and gate_pre.shape[1] >= H * Dv)
-    out = torch.empty((rows, H * Dv), dtype=_F32, device=proj.device)
+    if out is None:
+        out = torch.empty((rows, H * Dv), dtype=_F32, device=proj.device)
+    _f32(out)
+    assert out.shape[0] == rows and out.shape[1] >= H * Dv   # (a column slice of a wider buffer is fine)
     check(lib.mi_linear_attention(ptr(proj), proj.stride(0), q_off, k_off, v_off, int(acts[0]), int(acts[1]), int(acts[2]),
                                   int(decay_kind), ptr(decay), ptr(f_bias), ptr(lower), ptr(gate_pre),
                                   gate_pre.stride(0) if gate_pre is not None else 0, ptr(norm_w), int(norm_groups),
                                   ptr(state), ptr(cu_q), ptr(kv_lens), ptr(slot_ids), kv_lens.numel(), rows, H, D, Dv,
                                   float(eps), ptr(out), out.stride(0), stream()), "mi_linear_attention")
     return out
+
+
+# ---- looped pre-norm families: rotary positions with unit-normed heads, capped / head-mixed window attention beside a
+# retention, experts weighted on their input (csrc/seqmix.hip, csrc/gemm_any.hip)
+def gemm_any_grouped_glu(x, x_rows, w, w2, act: int, limit: float, row_scale, row_scale_rows, group_offsets, rows_max: int,
+                         y_rows, y_rows_total: int, exact: bool = False):
+    """gemm_any_grouped_act with a scale per sorted row on the accumulators (row_scale[row_scale_rows[m]]) and the limit
+    of ACT_CLAMPED_GLU."""
+    require_gpu(x, w, group_offsets)
+    _f32(x, row_scale)
+    _i32(x_rows, y_rows, group_offsets, row_scale_rows)
+    assert w.dim() == 3 and w.is_contiguous() and (w2 is None or (w2.shape == w.shape and w2.is_contiguous() and w2.dtype == w.dtype))
+    assert row_scale is None or row_scale.is_contiguous()
+    G, N, K = w.shape
+    assert x.shape[1] == K and group_offsets.numel() >= G + 1
+    y = torch.empty((y_rows_total, N), dtype=_F32, device=x.device)
+    check(lib.mi_gemm_any_grouped_glu(ptr(x), x.stride(0), ptr(x_rows), ptr(w), ptr(w2), _dt(w), int(act), float(limit),
+                                      ptr(row_scale), ptr(row_scale_rows), ptr(group_offsets), G, rows_max, ptr(y), N,
+                                      ptr(y_rows), N, K, int(exact), stream()), "mi_gemm_any_grouped_glu")
+    return y
+
+
+def rotary_store(proj, q_off: int, k_off: int, v_off: int, H: int, G: int, D: int, rot_dims: int, layout: int, inv_freq,
+                 amp: float, unit_norm: bool, eps: float, k_mult: float, cu_q, kv_lens, k_cache=None, v_cache=None, slots=None,
+                 block_size: int = 1) -> None:
+    """Rotates the H query and G key heads of every row of proj in place (see mi_rotary_store); with caches the key heads
+    go to k_cache [blocks, G, block_size, D] and the row's values at v_off to v_cache [blocks, Gv, block_size, Dv]."""
+    require_gpu(proj, k_cache, v_cache, slots)
+    _f32(proj, inv_freq)
+    _i32(cu_q, kv_lens, slots)
+    rows = proj.shape[0]
+    Gv = Dv = 0
+    dt = _C.DTYPE_F32
+    if k_cache is not None:
+        assert k_cache.is_contiguous() and k_cache.shape[1:] == (G, block_size, D), k_cache.shape
+        dt = _dt(k_cache)
+    if v_cache is not None:
+        assert v_cache.is_contiguous() and v_cache.shape[2] == block_size and (k_cache is None or v_cache.dtype == k_cache.dtype)
+        Gv, Dv = v_cache.shape[1], v_cache.shape[3]
+        dt = _dt(v_cache)
+    assert slots is None or slots.numel() == rows
+    assert rot_dims == 0 or (inv_freq.is_cuda and inv_freq.numel() >= rot_dims // 2)
+    check(lib.mi_rotary_store(ptr(proj), proj.stride(0), q_off, k_off, v_off, H, G, D, Gv, Dv, int(rot_dims), int(layout),
+                              ptr(inv_freq), float(amp), int(unit_norm), float(eps), float(k_mult), ptr(cu_q), ptr(kv_lens),
+                              kv_lens.numel(), ptr(k_cache), ptr(v_cache), dt, ptr(slots), rows, block_size, stream()),
+          "mi_rotary_store")
+
+
+def head_mix(o, talk, H: int, G: int, Dv: int, c0: int, n_chunk: int, out, out_scale: float = 1.0) -> None:
+    """out[:, h] = out_scale * sum_g talk[h, g] * o[:, g, (h // (H // G) - c0) * Dv : + Dv] for the heads whose key/value
+    head lies in [c0, c0 + n_chunk); o [rows, H * n_chunk * Dv], out [rows, >= H * Dv] (a column slice is fine)."""
+    require_gpu(o, talk, out)
+    _f32(o, talk, out)
+    rows = o.shape[0]
+    assert talk.shape == (H, H) and talk.is_contiguous() and o.shape[1] == H * n_chunk * Dv and out.shape[0] == rows
+    assert out.shape[1] >= H * Dv
+    check(lib.mi_head_mix(ptr(o), o.stride(0), ptr(talk), rows, H, G, Dv, c0, n_chunk, float(out_scale), ptr(out),
+                          out.stride(0), stream()), "mi_head_mix")
+
+
+def head_norm_gate(out, gate_pre, gate_act: int, norm_w, H: int, Dv: int, eps: float, out_scale: float = 1.0) -> None:
+    """out[:, h] <- out_scale * out[:, h] / rms (* norm_w) (* act(gate_pre[:, h])) per head, in place."""
+    require_gpu(out)
+    _f32(out, gate_pre, norm_w)
+    assert out.shape[1] >= H * Dv and (gate_pre is None or (gate_pre.shape[0] == out.shape[0] and gate_pre.shape[1] >= H * Dv))
+    assert norm_w is None or norm_w.numel() == Dv
+    check(lib.mi_head_norm_gate(ptr(out), out.stride(0), ptr(gate_pre), gate_pre.stride(0) if gate_pre is not None else 0,
+                                int(gate_act), ptr(norm_w), float(out_scale), out.shape[0], H, Dv, float(eps), stream()),
+          "mi_head_norm_gate")
