@@ -536,7 +536,7 @@ class RotaryWindowAttention(nn.Module):
         self.H, self.G, self.D, self.Dv = heads, kv_heads, dim, vdim
         self.window, self.scale, self.eps, self.unit_norm, self.softcap = window, scale, eps, unit_norm, softcap
         self.rot_dims = rot_dims
-        freq, self.rot_amp = rotary_table(rot_dims, rot_base, rot_scaling) if rot_dims else (torch.zeros(1), 1.0)
+        freq, self.rot_amp = rotary_table(rot_dims, rot_base, rot_scaling) if rot_dims else (torch.zeros(1, dtype=torch.float32), 1.0)
         self.register_buffer("inv_freq", freq, persistent=False)
         self.parts = {"q": heads * dim, "k": kv_heads * dim, "v": kv_heads * vdim}
         self.sink = _vector(heads) if sink else None
@@ -596,7 +596,7 @@ class Retention(nn.Module):
         super().__init__()
         assert len(decay) == heads and 0 <= rot_dims <= dim and rot_dims % 2 == 0
         self.H, self.D, self.Dv, self.eps, self.rot_dims = heads, dim, vdim, eps, rot_dims
-        freq, self.rot_amp = rotary_table(rot_dims, rot_base, rot_scaling) if rot_dims else (torch.zeros(1), 1.0)
+        freq, self.rot_amp = rotary_table(rot_dims, rot_base, rot_scaling) if rot_dims else (torch.zeros(1, dtype=torch.float32), 1.0)
         self.register_buffer("inv_freq", freq, persistent=False)
         self.register_buffer("decay", torch.tensor([float(d) for d in decay], dtype=torch.float64).to(torch.float32),
                              persistent=False)

@@ -288,6 +288,8 @@ def random_model(config, seed=0, overrides=None):
             t = torch.randn(shape, generator=g) * 0.1
         elif name == "embed":
             t = torch.randn(shape, generator=g) * 0.5
+        elif leaf in ("down", "o"):    # sublayer outputs well below the stream: an expert swapped at a router's near-tie
+            t = torch.randn(shape, generator=g) * ((0.15 if leaf == "down" else 0.4) * shape[-1] ** -0.5)   # (bf16 serving)
         else:
             t = torch.randn(shape, generator=g) * (1.5 * shape[-1] ** -0.5)
         out[name] = t.to(torch.bfloat16).to(torch.float32)
