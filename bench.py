@@ -503,11 +503,11 @@ def main():
                     help="N > 1: independent replicas (weak scaling, the headline value) AND tensor parallelism at the "
                          "fixed batch (reported under `tp_run` of the same line), or only one of the two")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--design", choices=("gazutar", "zedirax", "felolorn"), default=None,
+    ap.add_argument("--design", choices=("gazutar", "zedirax", "felolorn", "sanevik"), default=None,
                     help="instead of the headline workload: prefill / decode throughput of this model design beside the "
                          "closest existing model at equal size (nano-vllm-ascend_amd/bench/design_bench.py), one JSON line")
     ap.add_argument("--design-sizes", default="", help="with --design: comma-separated subset of its sizes")
-    ap.add_argument("--design-models", default="", help="with --design: comma-separated subset of felolorn,zedirax,gazutar,qwen3_moe")
+    ap.add_argument("--design-models", default="", help="with --design: comma-separated subset of sanevik,felolorn,zedirax,gazutar,qwen3_moe")
     args = ap.parse_args()
     if args.design is not None:
         sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "nano-vllm-ascend_amd", "bench"))

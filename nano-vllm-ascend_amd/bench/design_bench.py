@@ -1,5 +1,5 @@
 """Prefill and decode throughput of a model design beside the framework's closest existing model at equal size
-(`python bench.py --design gazutar | zedirax | felolorn`): random weights, layer sizes that resemble a real model's, both models through the same
+(`python bench.py --design gazutar | zedirax | felolorn | sanevik`): random weights, layer sizes that resemble a real model's, both models through the same
 engine entry points (add_request / step), each served the way the framework serves it (Qwen3-MoE: captured prefill and
 decode steps; Gazutar: what ModelRunner reports in `served_as`).
 
@@ -110,6 +110,49 @@ def felolorn_decode_weight_bytes(cfg: dict, batch: int) -> float:
     return 2.0 * (n + cfg["vocab"] * W)
 
 
+def sanevik_config(s: dict) -> dict:
+    """Sink attention / parallel (capped, head-mixed window attention beside a retention, half of the heads each) /
+    sink attention / parallel, the last two layers run twice (six layer runs per step, each with pages and state of its
+    own); every layer with a sparse feed-forward whose experts take their weight on the input."""
+    W, D, H, G = s["width"], s["dim"], s["heads"], s["kv_heads"]
+    att = {"type": "attention",
+           "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "mask": {"size": s["window"]}, "scale": 1.25 * D ** -0.5,
+                     "rot": {"base": 10000.0, "dims": D // 2,
+                             "scaling": {"factor": 4.0, "original": 4096, "fast": 16.0, "slow": 2.0}}}}
+    par = {"type": "parallel",
+           "mixer": {"left": {"heads": H // 2, "kv_heads": G // 2, "dim": D, "vdim": D, "mask": {"size": s["window"]},
+                              "scale": D ** -0.5, "softcap": 30.0, "conv": 4, "rot": {"base": 10000.0, "dims": D}},
+                     "right": {"heads": H // 2, "dim": D, "vdim": D, "rot": {"base": 100000.0, "dims": D // 2},
+                               "decay": [1.0 - 2.0 ** (-5 - 6 * h / H) for h in range(H // 2)]},
+                     "left_scale": 1.0, "right_scale": 0.5}}
+    moe = {"kind": "moe", "expert": {"ff": s["ff"], "limit": 7.0}, "router": {"experts": s["experts"], "top": s["top"]}}
+    order = [att, par]
+    n = s["layers"]
+    return {"architecture": "Sanevik", "vocab": s["vocab"], "width": W, "norm": {"eps": 1e-6},
+            "loop": {"start": n - 2, "stop": n, "times": 2}, "layers": [dict(order[i % 2], mlp=moe) for i in range(n)]}
+
+
+def sanevik_decode_weight_bytes(cfg: dict, batch: int) -> float:
+    """bf16 weight bytes one decode step of `batch` rows streams: every projection and the experts the rows can reach, once
+    per RUN of a layer (a looped layer's weights are read again in every pass), the tied table as the head."""
+    W, n = cfg["width"], 0
+    loop = cfg.get("loop") or {"start": 0, "stop": 0, "times": 1}
+    for i, l in enumerate(cfg["layers"]):
+        m = l["mixer"]
+        if l["type"] == "attention":
+            mix = W * (m["heads"] * m["dim"] + m["kv_heads"] * (m["dim"] + m["vdim"])) + m["heads"] * m["vdim"] * W
+        else:
+            a, r = m["left"], m["right"]
+            mix = W * (a["heads"] * a["dim"] + a["kv_heads"] * (a["dim"] + a["vdim"]) + 2 * r["heads"] * (r["dim"] + r["vdim"]))
+            mix += (a["heads"] * a["vdim"] + r["heads"] * r["vdim"]) * W
+        ml = l["mlp"]
+        if ml is not None:
+            hit = min(ml["router"]["experts"], batch * ml["router"]["top"])
+            mix += hit * 3 * W * ml["expert"]["ff"] + ml["router"]["experts"] * W
+        n += mix * (loop["times"] if loop["start"] <= i < loop["stop"] else 1)
+    return 2.0 * (n + cfg["vocab"] * W)
+
+
 def qwen3_moe_config(s: dict) -> dict:
     return dict(architectures=["Qwen3MoeForCausalLM"], model_type="qwen3_moe", hidden_size=s["width"],
                 num_hidden_layers=s["layers"], num_attention_heads=s["heads"], num_key_value_heads=s["kv_heads"],
@@ -187,6 +230,8 @@ def main(args) -> dict:
         return main_zedirax(args, batch, prompt_len)
     if design == "felolorn":
         return main_felolorn(args, batch, prompt_len)
+    if design == "sanevik":
+        return main_sanevik(args, batch, prompt_len)
     out = {"metric": "design_throughput", "design": "gazutar", "closest_model": "Qwen3MoeForCausalLM", "unit": "tokens/s",
            "dtype": "bf16", "data": "synthetic (random weights, random prompts)", "n_gpus": 1, "steps": args.steps,
            "warmup": args.warmup, "batch": batch, "prompt_len": prompt_len, "sizes": {}}
@@ -269,6 +314,43 @@ def main_felolorn(args, batch: int, prompt_len: int) -> dict:
         for other in ("zedirax", "gazutar"):
             if "felolorn" in entry and other in entry:
                 entry["felolorn_vs_" + other] = {k: entry["felolorn"][k] / entry[other][k] for k in ("prefill_tok_s", "decode_tok_s")}
+        out["sizes"][name] = entry
+    print(json.dumps(out), flush=True)
+    return out
+
+
+def main_sanevik(args, batch: int, prompt_len: int) -> dict:
+    """Sanevik beside Gazutar - the closest existing model: the same row-step engine path, fp32 residual, sliding-window
+    attention over paged K / V rows alternating with a matrix-state recurrence behind short convolutions, sparse
+    feed-forwards - at equal width, depth, heads, experts and vocabulary; Felolorn (sink softmax, head-decay linear
+    attention) and Qwen3-MoE at that size ride along (`--design-models` picks).  Sanevik runs its last two layers twice:
+    six layer runs per step against the others' four (`layer_runs` in the record)."""
+    out = {"metric": "design_throughput", "design": "sanevik", "closest_model": "Gazutar", "unit": "tokens/s",
+           "dtype": "bf16", "data": "synthetic (random weights, random prompts)", "n_gpus": 1, "steps": args.steps,
+           "warmup": args.warmup, "batch": batch, "prompt_len": prompt_len, "sizes": {}}
+    only_sizes = [x for x in getattr(args, "design_sizes", "").split(",") if x]
+    only_models = [x for x in getattr(args, "design_models", "").split(",") if x] or ["sanevik", "gazutar", "felolorn"]
+    for name, s in SIZES.items():
+        if only_sizes and name not in only_sizes:
+            continue
+        entry = {"shape": s}
+        sc, fc = sanevik_config(s), felolorn_config(s)
+        for label, cfg, wb, runs in (("sanevik", sc, sanevik_decode_weight_bytes(sc, batch), s["layers"] + 2),
+                                     ("gazutar", gazutar_config(s), decode_weight_bytes(s, batch, True), s["layers"]),
+                                     ("felolorn", fc, felolorn_decode_weight_bytes(fc, batch), s["layers"]),
+                                     ("qwen3_moe", qwen3_moe_config(s), decode_weight_bytes(s, batch, False), s["layers"])):
+            if label not in only_models:
+                continue
+            r = run_model(cfg, batch, prompt_len, args.steps, args.warmup)
+            r["layer_runs"] = runs
+            r["decode_weight_bytes"] = wb
+            r["decode_weight_roofline_frac"] = wb / (r["ms_per_decode_step"] * 1e-3) / HBM_BYTES_PER_S
+            entry[label] = r
+        for other in ("gazutar", "felolorn"):
+            if "sanevik" in entry and other in entry:
+                entry["sanevik_vs_" + other] = {k: entry["sanevik"][k] / entry[other][k] for k in ("prefill_tok_s", "decode_tok_s")}
+                entry["sanevik_vs_" + other + "_per_layer_run"] = {
+                    k: v * entry["sanevik"]["layer_runs"] / entry[other]["layer_runs"] for k, v in entry["sanevik_vs_" + other].items()}
         out["sizes"][name] = entry
     print(json.dumps(out), flush=True)
     return out
