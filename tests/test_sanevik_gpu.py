@@ -51,6 +51,7 @@ def mixed_replay(request, mixed_model):
     ("parallel_matrix_core_sizes", [with_mlp(parallel(heads=4, kv_heads=2, dim=64, vdim=32, dims=32, window=33, r_heads=2,
                                                       r_dim=64, r_vdim=64, r_dims=64), None)], {}),
     ("parallel_values_in_chunks", [with_mlp(parallel(heads=6, kv_heads=3, dim=16, vdim=112, dims=16), None)], {}),
+    ("parallel_values_in_chunks_off_16_bytes", [with_mlp(parallel(heads=6, kv_heads=3, dim=16, vdim=90, dims=16), None)], {}),
     ("parallel_one_kv_head_many_heads", [with_mlp(parallel(heads=10, kv_heads=1, dim=8, vdim=12, dims=4, r_heads=1, r_dim=130,
                                                            r_vdim=40, r_dims=130), None)], {}),
     ("parallel_no_decay_and_full_decay", [with_mlp(parallel(r_heads=2, decay=[1.0, 0.0]), None)], {}),
